@@ -1,0 +1,128 @@
+/*
+ * libna1d — 1-D neighbourhood attention (NA1D) for AMD MI355X (gfx950).
+ *
+ * C ABI of the shared library.  Every entry point takes raw device pointers,
+ * 64-bit sizes, a dtype tag and the HIP stream to launch on; it allocates
+ * nothing, keeps no global mutable state, is re-entrant, and returns an int
+ * status (NA1D_OK or a negative NA1D_ERR_* code) instead of asserting.  All
+ * tensors are dense and contiguous:
+ *
+ *   q, k, v, out, d*  : [B, T, C]  16-bit (bf16 or fp16 by `dtype`), C fastest,
+ *                       B = batch * heads (batch major, head minor)
+ *   attn, dattn       : [B, T, W]  fp32, slot j of query t addresses key t-left+j
+ *   keys outside [0,T) contribute exactly 0 (zero filled, never clamped/shifted)
+ *
+ * Limits: C % 8 == 0, 1 <= W <= 80, 0 <= left < W, B,T >= 1 (B == 0 or T == 0 is
+ * a no-op that returns NA1D_OK).  Pointers must be 16-byte aligned.
+ *
+ * The six un-fused entry points replace, one for one, the pybind functions of
+ * the reference extension (na1d_tensorcore/bf16_ana1d.cpp:8-104 and its fp16
+ * twin; the same six appear as torch.ops.na_cuda.* in
+ * pcf_nat_pytorch2.7.zip!/extension_na/na_cuda/csrc_tc240_or_bigger/main.cpp:27-41).
+ */
+#ifndef NA1D_H
+#define NA1D_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NA1D_BF16 0
+#define NA1D_FP16 1
+
+#define NA1D_OK               0
+#define NA1D_ERR_NULL        -1   /* a required pointer is NULL                      */
+#define NA1D_ERR_DTYPE       -2   /* dtype is neither NA1D_BF16 nor NA1D_FP16         */
+#define NA1D_ERR_HEAD_DIM    -3   /* C <= 0 or C % 8 != 0                             */
+#define NA1D_ERR_WINDOW      -4   /* W < 1, W > 80, left < 0 or left >= W             */
+#define NA1D_ERR_SHAPE       -5   /* negative B or T, B % H != 0, size overflow       */
+#define NA1D_ERR_ALIGN       -6   /* a tensor pointer is not 16-byte aligned          */
+#define NA1D_ERR_LAUNCH      -7   /* the HIP runtime rejected the launch              */
+#define NA1D_ERR_UNSUPPORTED -8   /* valid arguments that no built kernel covers      */
+
+#define NA1D_MAX_WINDOW 80
+
+/* Library version (major*10000 + minor*100 + patch) and message for a status. */
+int         na1d_version(void);
+const char *na1d_status_string(int status);
+
+/* P1 — band QK^T:  attn[b,t,j] = sum_c q[b,t,c] * k~[b,t-left+j,c].
+ * Replaces torch_ana_qk_forward (bf16_ana1d.cpp:8-27; kernels
+ * bf16_ana1d_kernel.cu:42-282). */
+int na1d_qk_forward(void *attn, const void *q, const void *k,
+                    int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+                    int dtype, void *stream);
+
+/* P2 — band times V:  out[b,t,c] = sum_j attn[b,t,j] * v~[b,t-left+j,c], fp32
+ * accumulate, round-to-nearest-even store.  Replaces torch_ana_av_forward
+ * (bf16_ana1d.cpp:57-69; kernel bf16_ana1d_kernel.cu:285-391). */
+int na1d_av_forward(void *out, const void *attn, const void *v,
+                    int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+                    int dtype, void *stream);
+
+/* dQ = P2(dattn, k).  Replaces torch_ana_q_backward (bf16_ana1d.cpp:29-41); the
+ * reference serves it with the same kernel as av_forward and so does this. */
+int na1d_q_backward(void *dq, const void *dattn, const void *k,
+                    int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+                    int dtype, void *stream);
+
+/* P3 — inverse-neighbourhood gather, no atomics:
+ *   dk[b,u,c] = sum_j dattn[b,u+left-j,j] * q[b,u+left-j,c]   (rows outside [0,T) dropped).
+ * Replaces torch_ana_k_backward (bf16_ana1d.cpp:43-55; kernel
+ * bf16_ana1d_kernel.cu:394-492). */
+int na1d_k_backward(void *dk, const void *dattn, const void *q,
+                    int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+                    int dtype, void *stream);
+
+/* dattn = P1(dout, v).  Replaces torch_ana_a_backward (bf16_ana1d.cpp:71-90). */
+int na1d_a_backward(void *dattn, const void *dout, const void *v,
+                    int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+                    int dtype, void *stream);
+
+/* dV = P3(attn, dout).  Replaces torch_ana_v_backward (bf16_ana1d.cpp:92-104). */
+int na1d_v_backward(void *dv, const void *attn, const void *dout,
+                    int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+                    int dtype, void *stream);
+
+/*
+ * Fused forward: QK^T -> (* scale) -> + rpb[h] -> + mask -> softmax -> . V, the
+ * [B,T,W] tensor never touching memory.  Replaces the sequence
+ * QK_Function -> +bias -> +mask -> softmax -> AV_Function of
+ * models/PCF_NATransformer.py:141-150 (mask of :87-99).
+ *
+ *   rpb      : fp32 [H, W] or NULL (no bias); head of row b is b % H
+ *   t_valid  : int32 [B / H] or NULL; valid length of each sample (T - padding).
+ *              A slot gets the additive -100 of the reference when its query
+ *              row t >= t_valid or its key lies outside [0, t_valid).
+ *   scale    : multiplies the fp32 scores (pass 1.0f when q is pre-scaled, as
+ *              the reference model does)
+ *   lse      : fp32 [B, T] out, log-sum-exp of each row's logits (for backward);
+ *              may be NULL for inference
+ */
+int na1d_fused_forward(void *out, float *lse,
+                       const void *q, const void *k, const void *v,
+                       const float *rpb, const int32_t *t_valid,
+                       int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
+                       float scale, int dtype, void *stream);
+
+/*
+ * Fused backward of the above.  Recomputes the probabilities from q, k, lse;
+ * replaces AV_Function.backward -> softmax backward -> QK_Function.backward
+ * (nattn.py:46-54,69-78).  dq is the gradient w.r.t. the q that was passed in
+ * (it already includes `scale`).
+ *
+ *   drpb : fp32 [H, W], ACCUMULATED into (caller zeroes it), or NULL to skip
+ */
+int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb,
+                        const void *q, const void *k, const void *v,
+                        const void *out, const void *dout, const float *lse,
+                        const float *rpb, const int32_t *t_valid,
+                        int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
+                        float scale, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NA1D_H */

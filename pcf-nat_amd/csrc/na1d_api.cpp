@@ -1,0 +1,136 @@
+// C ABI of libna1d: argument validation and dispatch.  No torch types, no
+// allocation, no global mutable state; kernels go to the stream that is passed in.
+#include "na1d_common.h"
+
+namespace {
+
+using na1d::Geom;
+
+inline bool misaligned(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+// Common checks of the un-fused entry points.  Returns NA1D_OK, an error, or
+// +1 for "nothing to do".
+int check(const void *o, const void *a, const void *b, int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+          int64_t H, int dtype, Geom &g) {
+    if (dtype != NA1D_BF16 && dtype != NA1D_FP16) return NA1D_ERR_DTYPE;
+    if (C <= 0 || C % 8 != 0 || C > (1 << 20)) return NA1D_ERR_HEAD_DIM;
+    if (W < 1 || W > NA1D_MAX_WINDOW || left < 0 || left >= W) return NA1D_ERR_WINDOW;
+    if (B < 0 || T < 0 || H < 1 || B % H != 0) return NA1D_ERR_SHAPE;
+    if (B == 0 || T == 0) return 1;
+    const int64_t widest = C > W ? C : W;
+    if (T > (INT64_MAX / 8) / widest || B > (INT64_MAX / 8) / (T * widest)) return NA1D_ERR_SHAPE;
+    if (!o || !a || !b) return NA1D_ERR_NULL;
+    if (misaligned(o) || misaligned(a) || misaligned(b)) return NA1D_ERR_ALIGN;
+    g.B = B;
+    g.T = T;
+    g.C = (int)C;
+    g.W = (int)W;
+    g.L = (int)left;
+    g.H = (int)H;
+    return NA1D_OK;
+}
+
+#define NA1D_CHECK(...)                     \
+    Geom g;                                 \
+    {                                       \
+        const int st = check(__VA_ARGS__);  \
+        if (st != NA1D_OK) return st > 0 ? NA1D_OK : st; \
+    }
+
+int band_qk(void *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s) {
+    const int st = na1d::mfma::qk((float *)attn, a, b, g, dtype, s);
+    return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::qk((float *)attn, a, b, g, dtype, s) : st;
+}
+int band_av(void *out, const void *attn, const void *v, const Geom &g, int dtype, hipStream_t s) {
+    const int st = na1d::mfma::av(out, (const float *)attn, v, g, dtype, s);
+    return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::av(out, (const float *)attn, v, g, dtype, s) : st;
+}
+int band_gather(void *out, const void *attn, const void *x, const Geom &g, int dtype, hipStream_t s) {
+    const int st = na1d::mfma::gather(out, (const float *)attn, x, g, dtype, s);
+    return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::gather(out, (const float *)attn, x, g, dtype, s) : st;
+}
+
+}  // namespace
+
+extern "C" {
+
+int na1d_version(void) { return 100; }
+
+const char *na1d_status_string(int status) {
+    switch (status) {
+        case NA1D_OK: return "ok";
+        case NA1D_ERR_NULL: return "a required pointer is NULL";
+        case NA1D_ERR_DTYPE: return "dtype must be NA1D_BF16 (0) or NA1D_FP16 (1)";
+        case NA1D_ERR_HEAD_DIM: return "head_dim must be a positive multiple of 8";
+        case NA1D_ERR_WINDOW: return "need 1 <= win_size <= 80 and 0 <= left < win_size";
+        case NA1D_ERR_SHAPE: return "bad B/T/H (negative, B not a multiple of H, or too large)";
+        case NA1D_ERR_ALIGN: return "tensor pointers must be 16-byte aligned";
+        case NA1D_ERR_LAUNCH: return "HIP rejected the kernel launch";
+        case NA1D_ERR_UNSUPPORTED: return "no kernel built for these arguments";
+        default: return "unknown status";
+    }
+}
+
+int na1d_qk_forward(void *attn, const void *q, const void *k, int64_t B, int64_t T, int64_t C, int64_t W,
+                    int64_t left, int dtype, void *stream) {
+    NA1D_CHECK(attn, q, k, B, T, C, W, left, 1, dtype, g);
+    return band_qk(attn, q, k, g, dtype, (hipStream_t)stream);
+}
+
+int na1d_a_backward(void *dattn, const void *dout, const void *v, int64_t B, int64_t T, int64_t C, int64_t W,
+                    int64_t left, int dtype, void *stream) {
+    NA1D_CHECK(dattn, dout, v, B, T, C, W, left, 1, dtype, g);
+    return band_qk(dattn, dout, v, g, dtype, (hipStream_t)stream);
+}
+
+int na1d_av_forward(void *out, const void *attn, const void *v, int64_t B, int64_t T, int64_t C, int64_t W,
+                    int64_t left, int dtype, void *stream) {
+    NA1D_CHECK(out, attn, v, B, T, C, W, left, 1, dtype, g);
+    return band_av(out, attn, v, g, dtype, (hipStream_t)stream);
+}
+
+int na1d_q_backward(void *dq, const void *dattn, const void *k, int64_t B, int64_t T, int64_t C, int64_t W,
+                    int64_t left, int dtype, void *stream) {
+    NA1D_CHECK(dq, dattn, k, B, T, C, W, left, 1, dtype, g);
+    return band_av(dq, dattn, k, g, dtype, (hipStream_t)stream);
+}
+
+int na1d_k_backward(void *dk, const void *dattn, const void *q, int64_t B, int64_t T, int64_t C, int64_t W,
+                    int64_t left, int dtype, void *stream) {
+    NA1D_CHECK(dk, dattn, q, B, T, C, W, left, 1, dtype, g);
+    return band_gather(dk, dattn, q, g, dtype, (hipStream_t)stream);
+}
+
+int na1d_v_backward(void *dv, const void *attn, const void *dout, int64_t B, int64_t T, int64_t C, int64_t W,
+                    int64_t left, int dtype, void *stream) {
+    NA1D_CHECK(dv, attn, dout, B, T, C, W, left, 1, dtype, g);
+    return band_gather(dv, attn, dout, g, dtype, (hipStream_t)stream);
+}
+
+int na1d_fused_forward(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+                       const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
+                       int64_t left, float scale, int dtype, void *stream) {
+    NA1D_CHECK(out, q, k, B, T, C, W, left, H, dtype, g);
+    if (!v) return NA1D_ERR_NULL;
+    if (misaligned(v)) return NA1D_ERR_ALIGN;
+    const int st = na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream);
+    if (st != NA1D_ERR_UNSUPPORTED) return st;
+    return na1d::generic::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream);
+}
+
+int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+                        const void *out, const void *dout, const float *lse, const float *rpb,
+                        const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
+                        int64_t left, float scale, int dtype, void *stream) {
+    NA1D_CHECK(dq, q, k, B, T, C, W, left, H, dtype, g);
+    if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
+    if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
+        return NA1D_ERR_ALIGN;
+    const int st = na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, scale, dtype,
+                                         (hipStream_t)stream);
+    if (st != NA1D_ERR_UNSUPPORTED) return st;
+    return na1d::generic::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, scale, dtype,
+                                    (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,104 @@
+// Shared device helpers for the NA1D kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "na1d.h"
+
+namespace na1d {
+
+constexpr float kMaskValue = -100.0f;   // additive mask of the reference model (models/PCF_NATransformer.py:98)
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// 16-bit element types.  Values travel as raw uint16_t; conversion is explicit.
+struct BF16 {
+    static constexpr int tag = NA1D_BF16;
+    __device__ static inline float to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+    // round to nearest even; NaN stays NaN
+    __device__ static inline uint16_t from_f32(float f) {
+        uint32_t u = __float_as_uint(f);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+};
+
+struct FP16 {
+    static constexpr int tag = NA1D_FP16;
+    __device__ static inline float to_f32(uint16_t h) {
+        _Float16 x;
+        __builtin_memcpy(&x, &h, 2);
+        return (float)x;
+    }
+    __device__ static inline uint16_t from_f32(float f) {
+        _Float16 x = (_Float16)f;   // v_cvt_f16_f32, round to nearest even
+        uint16_t h;
+        __builtin_memcpy(&h, &x, 2);
+        return h;
+    }
+};
+
+// Eight consecutive 16-bit channels = one 128-bit access.
+struct alignas(16) Chunk8 {
+    uint32_t w[4];
+};
+
+template <class DT>
+__device__ inline void unpack8(const Chunk8 &c, float (&f)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f[2 * i] = DT::to_f32((uint16_t)(c.w[i] & 0xffffu));
+        f[2 * i + 1] = DT::to_f32((uint16_t)(c.w[i] >> 16));
+    }
+}
+
+template <class DT>
+__device__ inline Chunk8 pack8(const float (&f)[8]) {
+    Chunk8 c;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        c.w[i] = (uint32_t)DT::from_f32(f[2 * i]) | ((uint32_t)DT::from_f32(f[2 * i + 1]) << 16);
+    return c;
+}
+
+__device__ inline float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+
+// Problem description shared by every launcher.
+struct Geom {
+    int64_t B, T;
+    int C, W, L;      // head_dim, window, left
+    int H;            // heads (B % H == 0); 1 for the un-fused entry points
+};
+
+// Host-side launch status check.
+inline int launch_status() { return hipGetLastError() == hipSuccess ? NA1D_OK : NA1D_ERR_LAUNCH; }
+
+// ---- generic (any C % 8 == 0, any W <= 80) kernels: na1d_generic.hip -------
+namespace generic {
+int qk(float *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s);
+int av(void *out, const float *attn, const void *v, const Geom &g, int dtype, hipStream_t s);
+int gather(void *out, const float *attn, const void *x, const Geom &g, int dtype, hipStream_t s);
+int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+              const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s);
+int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+              const void *out, const void *dout, const float *lse, const float *rpb,
+              const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s);
+}  // namespace generic
+
+// ---- MFMA kernels for the shapes they cover: na1d_mfma.hip ------------------
+// Same signatures; each returns NA1D_ERR_UNSUPPORTED when the shape is not
+// covered, and the caller then falls back to the generic kernel.
+namespace mfma {
+int qk(float *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s);
+int av(void *out, const float *attn, const void *v, const Geom &g, int dtype, hipStream_t s);
+int gather(void *out, const float *attn, const void *x, const Geom &g, int dtype, hipStream_t s);
+int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+              const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s);
+int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+              const void *out, const void *dout, const float *lse, const float *rpb,
+              const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s);
+}  // namespace mfma
+
+}  // namespace na1d

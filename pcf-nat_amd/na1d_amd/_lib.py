@@ -1,0 +1,107 @@
+"""ctypes binding of libna1d.so (the C ABI declared in include/na1d.h).
+
+The library is prebuilt in-tree (``pcf-nat_amd/lib/libna1d.so``); nothing is
+compiled at import.  There is no CPU fallback: if the library is missing or a
+call fails, a Python exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libna1d.so")
+
+BF16, FP16 = 0, 1
+
+_i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+
+_UNFUSED = ("na1d_qk_forward", "na1d_av_forward", "na1d_q_backward", "na1d_k_backward",
+            "na1d_a_backward", "na1d_v_backward")
+SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_version", "na1d_status_string")
+
+_lib = None
+
+
+class NA1DError(RuntimeError):
+    """A libna1d entry point returned a non-zero status."""
+
+
+def build_hint() -> str:
+    return ("libna1d.so not found at %s - build it with `make -C pcf-nat_amd/csrc` "
+            "(or `python -c 'import __graft_entry__ as g; g.build()'`)" % LIB_PATH)
+
+
+def load():
+    """Load (once) and return the ctypes handle; raises if the library is absent."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise NA1DError(build_hint())
+    lib = ctypes.CDLL(LIB_PATH)
+    for name in _UNFUSED:
+        f = getattr(lib, name)
+        f.restype = _int
+        f.argtypes = [_ptr, _ptr, _ptr, _i64, _i64, _i64, _i64, _i64, _int, _ptr]
+    lib.na1d_fused_forward.restype = _int
+    lib.na1d_fused_forward.argtypes = [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                       _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _ptr]
+    lib.na1d_fused_backward.restype = _int
+    lib.na1d_fused_backward.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _ptr]
+    lib.na1d_version.restype = _int
+    lib.na1d_version.argtypes = []
+    lib.na1d_status_string.restype = ctypes.c_char_p
+    lib.na1d_status_string.argtypes = [_int]
+    _lib = lib
+    return lib
+
+
+def dtype_tag(dtype: torch.dtype) -> int:
+    if dtype == torch.bfloat16:
+        return BF16
+    if dtype == torch.float16:
+        return FP16
+    raise TypeError("NA1D supports torch.bfloat16 and torch.float16, got %s" % dtype)
+
+
+def _stream(t: torch.Tensor):
+    if t.device.type != "cuda":
+        raise NA1DError("NA1D tensors must live on the GPU (got device %s); there is no CPU path" % t.device)
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _p(t):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+def check(status: int, name: str):
+    if status != 0:
+        raise NA1DError("%s failed: %s (status %d)" % (name, load().na1d_status_string(status).decode(), status))
+
+
+def call_unfused(name: str, out, a, b, B, T, C, W, left, dtype):
+    """``name(out, a, b, B, T, C, W, left, dtype, stream)`` on torch's current stream."""
+    lib = load()
+    with torch.cuda.device(out.device):
+        st = getattr(lib, name)(_p(out), _p(a), _p(b), B, T, C, W, left, dtype_tag(dtype), _stream(out))
+    check(st, name)
+
+
+def call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, H, T, C, W, left, scale):
+    lib = load()
+    with torch.cuda.device(out.device):
+        st = lib.na1d_fused_forward(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid),
+                                    B, H, T, C, W, left, scale, dtype_tag(q.dtype), _stream(out))
+    check(st, "na1d_fused_forward")
+
+
+def call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, B, H, T, C, W, left, scale):
+    lib = load()
+    with torch.cuda.device(dq.device):
+        st = lib.na1d_fused_backward(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(out), _p(dout),
+                                     _p(lse), _p(rpb), _p(t_valid), B, H, T, C, W, left, scale,
+                                     dtype_tag(q.dtype), _stream(dq))
+    check(st, "na1d_fused_backward")

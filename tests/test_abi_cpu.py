@@ -1,0 +1,110 @@
+"""CPU-side checks of the C-ABI library: it loads, exports every symbol the
+header declares, and validates arguments before touching the GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from na1d_amd import _lib, nattn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "na1d.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(na1d_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 10
+    for name in names:
+        assert hasattr(lib, name), name
+    assert set(_lib.SYMBOLS) <= set(names)
+    assert lib.na1d_version() >= 100
+
+
+def test_status_strings():
+    lib = _lib.load()
+    assert lib.na1d_status_string(0) == b"ok"
+    for code in range(-8, 0):
+        assert len(lib.na1d_status_string(code)) > 3
+    assert lib.na1d_status_string(-99) == b"unknown status"
+
+
+def _call(lib, name, o, a, b, B, T, C, W, left, dtype):
+    P = ctypes.c_void_p
+    return getattr(lib, name)(P(o), P(a), P(b), B, T, C, W, left, dtype, None)
+
+
+@pytest.mark.parametrize("name", ["na1d_qk_forward", "na1d_av_forward", "na1d_q_backward",
+                                  "na1d_k_backward", "na1d_a_backward", "na1d_v_backward"])
+def test_argument_validation_happens_before_any_launch(name):
+    """Bad arguments come back as status codes (the reference has no checks at
+    all: bad shapes are silent out-of-bounds there).  0x1000 is a fake aligned
+    address: validation must reject before it is ever dereferenced."""
+    lib = _lib.load()
+    ok = 0x1000
+    assert _call(lib, name, ok, ok, ok, 2, 8, 12, 5, 2, 0) == -3      # C % 8
+    assert _call(lib, name, ok, ok, ok, 2, 8, 0, 5, 2, 0) == -3
+    assert _call(lib, name, ok, ok, ok, 2, 8, 16, 81, 2, 0) == -4     # W > 80
+    assert _call(lib, name, ok, ok, ok, 2, 8, 16, 0, 0, 0) == -4
+    assert _call(lib, name, ok, ok, ok, 2, 8, 16, 5, 5, 0) == -4      # left >= W
+    assert _call(lib, name, ok, ok, ok, 2, 8, 16, 5, -1, 0) == -4
+    assert _call(lib, name, ok, ok, ok, 2, 8, 16, 5, 2, 7) == -2      # dtype
+    assert _call(lib, name, ok, ok, ok, -1, 8, 16, 5, 2, 0) == -5
+    assert _call(lib, name, ok, ok, ok, 1 << 40, 1 << 40, 16, 5, 2, 0) == -5   # overflow
+    assert _call(lib, name, None, ok, ok, 2, 8, 16, 5, 2, 0) == -1
+    assert _call(lib, name, ok, None, ok, 2, 8, 16, 5, 2, 0) == -1
+    assert _call(lib, name, ok, ok, ok + 2, 2, 8, 16, 5, 2, 0) == -6   # alignment
+    # empty problems are a no-op, even with null pointers
+    assert _call(lib, name, None, None, None, 0, 8, 16, 5, 2, 0) == 0
+    assert _call(lib, name, None, None, None, 2, 0, 16, 5, 2, 1) == 0
+
+
+def test_fused_entry_points_validate():
+    lib = _lib.load()
+    P = ctypes.c_void_p
+    ok = P(0x1000)
+    f = lib.na1d_fused_forward
+    assert f(ok, None, ok, ok, ok, None, None, 4, 3, 8, 16, 5, 2, 1.0, 0, None) == -5   # B % H
+    assert f(ok, None, ok, ok, None, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, None) == -1  # v missing
+    assert f(ok, None, ok, ok, ok, None, None, 4, 2, 8, 20, 5, 2, 1.0, 0, None) == -3
+    assert f(None, None, None, None, None, None, None, 0, 1, 8, 16, 5, 2, 1.0, 0, None) == 0
+    b = lib.na1d_fused_backward
+    assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, None, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, None) == -1  # lse
+    assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 90, 2, 1.0, 0, None) == -4
+
+
+def test_python_layer_mirrors_reference_entry_points():
+    """Names, dispatch and asserts of na1d_tensorcore/nattn.py:128-137."""
+    qk, av = nattn.getNA1dFunction(C=16, dilation=1, dtype=torch.bfloat16)
+    assert (qk.__name__, av.__name__) == ("bf16_ANA1d_QK_Function", "bf16_ANA1d_AV_Function")
+    qk, av = nattn.getNA1dFunction(C=32, dilation=1, dtype=torch.float16)
+    assert (qk.__name__, av.__name__) == ("fp16_ANA1d_QK_Function", "fp16_ANA1d_AV_Function")
+    assert issubclass(qk, torch.autograd.Function) and issubclass(av, torch.autograd.Function)
+    with pytest.raises(AssertionError):
+        nattn.getNA1dFunction(C=12, dilation=1, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        nattn.getNA1dFunction(C=16, dilation=2, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        nattn.getNA1dFunction(C=16, dilation=1, dtype=torch.float32)
+    import na1d_tensorcore.nattn as shim      # the import path the reference models use
+    assert shim.getNA1dFunction is nattn.getNA1dFunction
+
+
+def test_no_cpu_fallback():
+    """CPU tensors are refused loudly; nothing routes through the oracle."""
+    qk, _ = nattn.getNA1dFunction(C=8, dilation=1, dtype=torch.bfloat16)
+    q = torch.zeros(1, 4, 8, dtype=torch.bfloat16)
+    with pytest.raises(Exception):
+        qk.apply(q, q, 3, 1, 1)
+    src = open(os.path.join(ROOT, "pcf-nat_amd", "na1d_amd", "_lib.py")).read()
+    for mod in ("nattn.py", "fused.py", "_lib.py", "__init__.py"):
+        text = open(os.path.join(ROOT, "pcf-nat_amd", "na1d_amd", mod)).read()
+        assert "oracle" not in text.replace("no CPU path", "")
+    assert "CDLL" in src

@@ -1,0 +1,262 @@
+"""GPU parity: the HIP path (called through the C ABI) against the CPU oracle on
+the same seeded inputs.  Tolerances are the contract's: relative L2 error
+<= 1e-2 for bf16 and <= 2e-3 for fp16 on outputs and gradients; integer-like
+facts (zero fill, shifts, aliasing) are checked bit for bit."""
+import os
+
+import pytest
+import torch
+
+from oracle import na1d_oracle as O
+from na1d_amd import _lib, nattn, na1d_fused
+from na1d_amd.fused import na1d_fused_forward_lse
+from _util import TOL, dev, make_inputs, seeded_scores
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.bfloat16, torch.float16]
+
+# (B, T, C, W, left): edge geometry the reference's CPU branch defines -
+# T < W, even W, left = 0, left = W-1, W = 1, W = 80, T = 1, odd head_dim multiples
+SHAPES = [
+    (2, 9, 8, 5, 2), (2, 9, 16, 4, 1), (3, 7, 8, 1, 0), (2, 3, 16, 7, 3), (2, 2, 8, 5, 0),
+    (2, 5, 8, 5, 4), (1, 1, 8, 3, 1), (2, 40, 24, 11, 5), (2, 33, 40, 8, 3), (1, 100, 16, 27, 13),
+    (2, 100, 128, 80, 39), (2, 17, 16, 80, 0), (2, 130, 64, 7, 3), (4, 300, 32, 15, 7), (3, 65, 16, 27, 26),
+    (2, 47, 48, 33, 16), (2, 64, 16, 27, 13), (1, 16, 32, 15, 7), (2, 15, 64, 7, 3), (2, 250, 16, 9, 8),
+]
+
+
+def _unfused(name, out, a, b, W, left):
+    B, T, C = (a if a.dtype != torch.float32 else b).shape
+    _lib.call_unfused(name, out, a, b, B, T, C, W, left, (a if a.dtype != torch.float32 else b).dtype)
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_unfused_primitives(shape, dtype):
+    B, T, C, W, L = shape
+    q, k, v = make_inputs(B, T, C, W, seed=sum(shape), dtype=dtype)
+    s = seeded_scores(B, T, W, seed=7)
+    qd, kd, vd, sd = dev(q, k, v, s)
+    tol = TOL[dtype]
+
+    attn = _unfused("na1d_qk_forward", torch.empty(B, T, W, device="cuda"), qd, kd, W, L)
+    want = O.qk_band(q.float(), k.float(), W, L)
+    assert O.rel_l2(attn, want) < 1e-5, "P1"
+    # zero fill is exact
+    assert (attn.cpu()[want == 0] == 0).all()
+
+    out = _unfused("na1d_av_forward", torch.empty_like(vd), sd, vd, W, L)
+    assert O.rel_l2(out.float(), O.av_band(s, v.float(), W, L)) < tol, "P2"
+
+    dk = _unfused("na1d_k_backward", torch.empty_like(qd), sd, qd, W, L)
+    assert O.rel_l2(dk.float(), O.inverse_gather(s, q.float(), W, L)) < tol, "P3"
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_aliasing_identities_bit_for_bit(dtype):
+    """bf16_ana1d.cpp:57-104: av_forward == q_backward, a_backward == qk_forward on
+    (dO, v), v_backward == k_backward on (P, dO)."""
+    B, T, C, W, L = 4, 77, 32, 15, 7
+    x, y, _ = make_inputs(B, T, C, W, 5, dtype)
+    s = seeded_scores(B, T, W, 5)
+    xd, yd, sd = dev(x, y, s)
+    e16 = lambda: torch.empty_like(xd)
+    e32 = lambda: torch.empty(B, T, W, device="cuda")
+    assert torch.equal(_unfused("na1d_av_forward", e16(), sd, yd, W, L), _unfused("na1d_q_backward", e16(), sd, yd, W, L))
+    assert torch.equal(_unfused("na1d_a_backward", e32(), xd, yd, W, L), _unfused("na1d_qk_forward", e32(), xd, yd, W, L))
+    assert torch.equal(_unfused("na1d_v_backward", e16(), sd, xd, W, L), _unfused("na1d_k_backward", e16(), sd, xd, W, L))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_one_hot_probabilities_shift_values_exactly(dtype):
+    B, T, C, W, L = 2, 50, 16, 7, 3
+    _, _, v = make_inputs(B, T, C, W, 11, dtype)
+    vd = dev(v)
+    for j0 in (0, 3, 6):
+        p = torch.zeros(B, T, W)
+        p[:, :, j0] = 1
+        out = _unfused("na1d_av_forward", torch.empty_like(vd), p.cuda(), vd, W, L).cpu()
+        want = torch.zeros_like(v)
+        lo, hi = max(0, L - j0), min(T, T + L - j0)
+        want[:, lo:hi] = v[:, lo - L + j0:hi - L + j0]
+        assert torch.equal(out, want)
+
+
+def _reference_style_chain(QK, AV, q, k, v, rpb, mask, H, W, L):
+    """The CUDA branch of models/PCF_NATransformer.py:141-150 with our Functions."""
+    B, T, _ = q.shape
+    attn = QK.apply(q, k, W, L, 1)
+    attn = attn.view(B // H, H, T, W) + rpb.view(1, H, 1, W)
+    attn = attn + mask.unsqueeze(1)
+    attn = torch.softmax(attn.view(B, T, W), dim=-1)
+    return AV.apply(attn, v, W, L, 1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", [(2, 4, 60, 16, 27, 13), (3, 2, 33, 32, 15, 7), (2, 2, 9, 64, 7, 3), (2, 3, 21, 24, 8, 3)],
+                         ids=lambda g: "x".join(map(str, g)))
+def test_dropin_autograd_chain_matches_oracle(geom, dtype):
+    N, H, T, C, W, L = geom
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, W, 21, dtype, n=4, scale=C ** -0.5)
+    g = torch.Generator().manual_seed(3)
+    rpb = torch.randn(H, W, generator=g) * 0.5
+    pad = torch.tensor([0] + [T // 3] * (N - 1))
+    QK, AV = nattn.getNA1dFunction(C, 1, dtype)
+
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    rd = rpb.cuda().requires_grad_(True)
+    mask = O.attn_mask(T, W, L, pad).cuda()
+    out = _reference_style_chain(QK, AV, qd, kd, vd, rd, mask, H, W, L)
+    out.backward(do.cuda())
+
+    want_o, _, _ = O.na1d_forward(q.float(), k.float(), v.float(), W, L, rpb, pad, H)
+    wq, wk, wv, wr = O.na1d_backward(q.float(), k.float(), v.float(), do.float(), W, L, rpb, pad, H)
+    tol = TOL[dtype]
+    assert out.dtype == dtype and qd.grad.dtype == dtype
+    assert O.rel_l2(out.float(), want_o) < tol
+    assert O.rel_l2(qd.grad.float(), wq) < tol
+    assert O.rel_l2(kd.grad.float(), wk) < tol
+    assert O.rel_l2(vd.grad.float(), wv) < tol
+    assert O.rel_l2(rd.grad, wr) < tol
+
+
+FUSED_GEOMS = [  # (N, H, T, C, W, left)
+    (2, 4, 60, 16, 27, 13), (3, 2, 33, 32, 15, 7), (2, 2, 9, 64, 7, 3), (2, 3, 21, 24, 8, 3), (1, 1, 1, 8, 3, 1),
+    (2, 2, 5, 16, 27, 13), (1, 2, 100, 16, 27, 0), (1, 2, 100, 16, 27, 26), (2, 1, 70, 40, 80, 40), (2, 16, 100, 16, 27, 13),
+    (3, 4, 150, 16, 27, 13), (2, 8, 300, 32, 15, 7), (4, 4, 200, 64, 7, 3), (1, 2, 129, 128, 5, 2), (2, 2, 48, 16, 1, 0),
+    (1, 4, 257, 32, 40, 7), (1, 2, 31, 64, 33, 20),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", FUSED_GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_fused_forward_backward_matches_oracle(geom, dtype):
+    N, H, T, C, W, L = geom
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, W, 31, dtype, n=4, scale=C ** -0.5)
+    g = torch.Generator().manual_seed(4)
+    rpb = torch.randn(H, W, generator=g) * 0.5
+    pad = torch.tensor([0, T // 2, T][:N] + [1] * max(0, N - 3))
+    t_valid = (T - pad).to(torch.int32)
+
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    rd = rpb.cuda().requires_grad_(True)
+    out = na1d_fused(qd, kd, vd, W, L, rpb=rd, t_valid=t_valid.cuda(), num_heads=H)
+    out.backward(do.cuda())
+
+    qf, kf, vf = q.float(), k.float(), v.float()
+    want_o, _, want_lse = O.na1d_forward(qf, kf, vf, W, L, rpb, pad, H)
+    wq, wk, wv, wr = O.na1d_backward(qf, kf, vf, do.float(), W, L, rpb, pad, H)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float(), want_o) < tol, "O"
+    assert O.rel_l2(qd.grad.float(), wq) < tol, "dQ"
+    assert O.rel_l2(kd.grad.float(), wk) < tol, "dK"
+    assert O.rel_l2(vd.grad.float(), wv) < tol, "dV"
+    assert O.rel_l2(rd.grad, wr) < tol, "drpb"
+    _, lse = na1d_fused_forward_lse(qd.detach(), kd.detach(), vd.detach(), W, L, rd.detach(), t_valid.cuda(), H)
+    assert torch.allclose(lse.cpu(), want_lse, atol=2e-3, rtol=1e-4), "LSE"
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_fused_scale_argument_and_optional_inputs(dtype):
+    """scale multiplies the fp32 scores; rpb / t_valid / lse are optional."""
+    N, H, T, C, W, L = 2, 2, 40, 32, 15, 7
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, W, 41, dtype, n=4)
+    scale = C ** -0.5
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = na1d_fused(qd, kd, vd, W, L, scale=scale)
+    out.backward(do.cuda())
+    qs = (q.float() * scale).requires_grad_(True)
+    want_o, _, _ = O.na1d_forward(qs, k.float(), v.float(), W, L)
+    wq, wk, wv, _ = O.na1d_backward(q.float() * scale, k.float(), v.float(), do.float(), W, L)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float(), want_o) < tol
+    assert O.rel_l2(qd.grad.float(), wq * scale) < tol      # chain rule through q*scale
+    assert O.rel_l2(kd.grad.float(), wk) < tol
+    assert O.rel_l2(vd.grad.float(), wv) < tol
+    # lse = NULL is allowed for inference
+    o2 = torch.empty_like(qd)
+    _lib.call_fused_forward(o2, None, qd.detach(), kd.detach(), vd.detach(), None, None, B, 1, T, C, W, L, scale)
+    assert torch.equal(o2, out.detach())
+
+
+def test_config1_forward_bf16():
+    """Single NA1D forward, bf16: batch 32, heads 4, T 200, head_dim 64, window 7."""
+    N, H, T, C, W = 32, 4, 200, 64, 7
+    _, L = O.split_window(W)
+    q, k, v = make_inputs(N * H, T, C, W, 1, torch.bfloat16, scale=C ** -0.5)
+    out = na1d_fused(*dev(q, k, v), W, L, num_heads=H)
+    want, _, _ = O.na1d_forward(q.float(), k.float(), v.float(), W, L)
+    assert O.rel_l2(out.float(), want) < 1e-2
+    QK, AV = nattn.getNA1dFunction(C, 1, torch.bfloat16)
+    qd, kd, vd = dev(q, k, v)
+    out2 = AV.apply(torch.softmax(QK.apply(qd, kd, W, L, 1) + O.attn_mask(T, W, L).cuda(), -1), vd, W, L, 1)
+    assert O.rel_l2(out2.float(), want) < 1e-2
+
+
+def test_config2_forward_backward_fp16():
+    """NA1D fwd+bwd, fp16: batch 128, heads 8, T 300, head_dim 32, window 15; dQ/dK/dV vs fp32."""
+    N, H, T, C, W = 128, 8, 300, 32, 15
+    _, L = O.split_window(W)
+    q, k, v, do = make_inputs(N * H, T, C, W, 2, torch.float16, n=4, scale=C ** -0.5)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = na1d_fused(qd, kd, vd, W, L, num_heads=H)
+    out.backward(do.cuda())
+    torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
+    qf, kf, vf = q.float(), k.float(), v.float()
+    want, _, _ = O.na1d_forward(qf, kf, vf, W, L)
+    wq, wk, wv, _ = O.na1d_backward_formulas(qf, kf, vf, do.float(), W, L)
+    for name, got, ref in (("O", out, want), ("dQ", qd.grad, wq), ("dK", kd.grad, wk), ("dV", vd.grad, wv)):
+        assert O.rel_l2(got.float(), ref) < 2e-3, name
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_model_shape_properties_at_full_size(dtype):
+    """cfg3's NA shape (B 4096, T 100, C 16, W 27): size-independent properties
+    instead of a full CPU oracle pass - batch invariance, agreement of the fused
+    kernel with the un-fused chain, rows of P summing to one via v = 1."""
+    N, H, T, C, W, L = 256, 16, 100, 16, 27, 13
+    B = N * H
+    q, k, v = make_inputs(B, T, C, W, 51, dtype, scale=0.25)
+    qd, kd, vd = dev(q, k, v)
+    out = na1d_fused(qd, kd, vd, W, L, num_heads=H)
+    # a slice alone gives the same bits as inside the batch
+    sl = slice(1000, 1016)
+    out_sl = na1d_fused(qd[sl].contiguous(), kd[sl].contiguous(), vd[sl].contiguous(), W, L, num_heads=H)
+    assert torch.equal(out[sl], out_sl)
+    # the slice against the oracle
+    want, _, _ = O.na1d_forward(q[sl].float(), k[sl].float(), v[sl].float(), W, L)
+    assert O.rel_l2(out_sl.float(), want) < TOL[dtype]
+    # fused == un-fused chain (two independent kernel families)
+    QK, AV = nattn.getNA1dFunction(C, 1, dtype)
+    chain = AV.apply(torch.softmax(QK.apply(qd, kd, W, L, 1) + O.attn_mask(T, W, L).cuda(), -1), vd, W, L, 1)
+    assert O.rel_l2(out.float(), chain.float()) < TOL[dtype]
+    # v = 1 -> every output element is sum_j P = 1 (up to e^-100 on masked slots)
+    ones = na1d_fused(qd, kd, torch.ones_like(vd), W, L, num_heads=H)
+    assert (ones.float() - 1).abs().max().item() < (2e-2 if dtype == torch.bfloat16 else 4e-3)
+
+
+def test_runs_on_the_current_stream():
+    """Launches go to torch's current stream (the reference uses the legacy default
+    stream; its data prefetcher runs a side stream, public/Utils.py:89-100)."""
+    B, T, C, W, L = 8, 120, 16, 27, 13
+    q, k, v = dev(*make_inputs(B, T, C, W, 61, torch.bfloat16))
+    base = na1d_fused(q, k, v, W, L)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        other = na1d_fused(q, k, v, W, L)
+    side.synchronize()
+    assert torch.equal(base, other)
+
+
+def test_errors_become_python_exceptions():
+    q = torch.zeros(2, 8, 16, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.NA1DError):
+        _lib.call_unfused("na1d_qk_forward", torch.empty(2, 8, 81, device="cuda"), q, q, 2, 8, 16, 81, 3, q.dtype)
+    with pytest.raises(_lib.NA1DError):
+        _lib.call_unfused("na1d_qk_forward", torch.empty(2, 8, 5, device="cuda"), q, q, 2, 8, 12, 5, 2, q.dtype)

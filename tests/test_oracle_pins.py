@@ -1,0 +1,261 @@
+"""Pins for the CPU oracle: every check here is chosen so that a plausible
+mistake in oracle/na1d_oracle.py (dropped term, wrong sign, shifted or clamped
+window, transposed operand) fails it.  None of them re-types the oracle's
+formula; they use brute-force index loops, library routines on special cases,
+closed forms and algebraic identities."""
+import itertools
+import math
+
+import pytest
+import torch
+
+from oracle import na1d_oracle as O
+
+torch.manual_seed(0)
+F64 = torch.float64
+
+GEOMS = [  # (T, W, left)
+    (9, 5, 2), (9, 4, 1), (9, 4, 2), (7, 1, 0), (3, 7, 3), (2, 5, 0), (5, 5, 4), (1, 3, 1), (6, 11, 5),
+]
+
+
+def _rand(*shape):
+    return torch.randn(*shape, dtype=F64)
+
+
+# ---------------------------------------------------------------- brute force
+def _brute_p1(q, k, W, L, d=1):
+    B, T, C = q.shape
+    s = torch.zeros(B, T, W, dtype=q.dtype)
+    for b, t, j in itertools.product(range(B), range(T), range(W)):
+        u = t + (j - L) * d
+        if 0 <= u < T:
+            s[b, t, j] = sum(q[b, t, c] * k[b, u, c] for c in range(C))
+    return s
+
+
+def _brute_p2(p, v, W, L, d=1):
+    B, T, C = v.shape
+    o = torch.zeros(B, T, C, dtype=v.dtype)
+    for b, t, j in itertools.product(range(B), range(T), range(W)):
+        u = t + (j - L) * d
+        if 0 <= u < T:
+            o[b, t] += p[b, t, j] * v[b, u]
+    return o
+
+
+def _brute_p3(s, x, W, L, d=1):
+    """Gather form, as the reference kernel indexes it (.cu:457-459)."""
+    B, T, C = x.shape
+    o = torch.zeros(B, T, C, dtype=x.dtype)
+    for b, u, j in itertools.product(range(B), range(T), range(W)):
+        t = u - (j - L) * d
+        if 0 <= t < T:
+            o[b, u] += s[b, t, j] * x[b, t]
+    return o
+
+
+@pytest.mark.parametrize("T,W,L", GEOMS)
+def test_primitives_match_brute_force(T, W, L):
+    q, k, v = _rand(2, T, 8), _rand(2, T, 8), _rand(2, T, 8)
+    s = _rand(2, T, W)
+    assert torch.allclose(O.qk_band(q, k, W, L), _brute_p1(q, k, W, L), atol=1e-12)
+    assert torch.allclose(O.av_band(s, v, W, L), _brute_p2(s, v, W, L), atol=1e-12)
+    assert torch.allclose(O.inverse_gather(s, q, W, L), _brute_p3(s, q, W, L), atol=1e-12)
+
+
+@pytest.mark.parametrize("d", [2, 3])
+def test_dilated_primitives_match_brute_force(d):
+    T, W, L = 11, 5, 2
+    q, k, v, s = _rand(1, T, 8), _rand(1, T, 8), _rand(1, T, 8), _rand(1, T, W)
+    assert torch.allclose(O.qk_band(q, k, W, L, d), _brute_p1(q, k, W, L, d), atol=1e-12)
+    assert torch.allclose(O.av_band(s, v, W, L, d), _brute_p2(s, v, W, L, d), atol=1e-12)
+    assert torch.allclose(O.inverse_gather(s, q, W, L, d), _brute_p3(s, q, W, L, d), atol=1e-12)
+
+
+# ---------------------------------------------------------------- special cases → library routines
+def test_p1_w1_is_rowwise_dot():
+    q, k = _rand(3, 10, 16), _rand(3, 10, 16)
+    assert torch.allclose(O.qk_band(q, k, 1, 0)[..., 0], (q * k).sum(-1), atol=1e-12)
+
+
+def test_p1_full_window_contains_dense_matmul():
+    """L=T-1, W=2T-1: S[t, u-t+L] = (q @ k^T)[t,u] for every (t,u); the rest is 0."""
+    T = 6
+    q, k = _rand(2, T, 8), _rand(2, T, 8)
+    L, W = T - 1, 2 * T - 1
+    s = O.qk_band(q, k, W, L)
+    dense = q @ k.transpose(1, 2)
+    seen = torch.zeros_like(s, dtype=torch.bool)
+    for t in range(T):
+        for u in range(T):
+            assert torch.allclose(s[:, t, u - t + L], dense[:, t, u], atol=1e-12)
+            seen[:, t, u - t + L] = True
+    assert (s[~seen] == 0).all()
+
+
+def test_p1_k_ones_counts_zero_fill_not_clamping():
+    """k = 1: S[t,j] = sum_c q[t,c] where the key exists and exactly 0 elsewhere;
+    a clamped or shifted (NATTEN-style) window would give non-zero edge slots."""
+    T, W, L = 8, 5, 2
+    q = _rand(1, T, 8)
+    s = O.qk_band(q, torch.ones(1, T, 8, dtype=F64), W, L)
+    for t in range(T):
+        for j in range(W):
+            inside = 0 <= t - L + j < T
+            want = q[0, t].sum() if inside else torch.tensor(0.0, dtype=F64)
+            assert torch.allclose(s[0, t, j], want, atol=1e-12)
+    assert (s[0, 0, :L] == 0).all() and (s[0, T - 1, L + 1:] == 0).all()
+
+
+def test_p2_one_hot_is_exact_shift():
+    T, W, L, C = 9, 5, 2, 8
+    v = _rand(2, T, C)
+    for j0 in range(W):
+        p = torch.zeros(2, T, W, dtype=F64)
+        p[:, :, j0] = 1
+        o = O.av_band(p, v, W, L)
+        for t in range(T):
+            u = t - L + j0
+            want = v[:, u] if 0 <= u < T else torch.zeros(2, C, dtype=F64)
+            assert torch.equal(o[:, t], want)
+
+
+def test_p2_uniform_probabilities_do_not_renormalise():
+    T, W, L, C = 10, 7, 3, 8
+    o = O.av_band(torch.full((1, T, W), 1.0 / W, dtype=F64), torch.full((1, T, C), 2.5, dtype=F64), W, L)
+    for t in range(T):
+        n_valid = sum(0 <= t - L + j < T for j in range(W))
+        assert torch.allclose(o[0, t], torch.full((C,), 2.5 * n_valid / W, dtype=F64), atol=1e-12)
+
+
+# ---------------------------------------------------------------- adjoint identities
+@pytest.mark.parametrize("T,W,L", GEOMS)
+def test_adjoint_identities(T, W, L):
+    q, k, v = _rand(2, T, 8), _rand(2, T, 8), _rand(2, T, 8)
+    G, P, GO = _rand(2, T, W), _rand(2, T, W), _rand(2, T, 8)
+    a = (O.qk_band(q, k, W, L) * G).sum()
+    assert torch.allclose(a, (q * O.av_band(G, k, W, L)).sum(), atol=1e-10)
+    assert torch.allclose(a, (k * O.inverse_gather(G, q, W, L)).sum(), atol=1e-10)
+    b = (O.av_band(P, v, W, L) * GO).sum()
+    assert torch.allclose(b, (P * O.qk_band(GO, v, W, L)).sum(), atol=1e-10)
+    assert torch.allclose(b, (v * O.inverse_gather(P, GO, W, L)).sum(), atol=1e-10)
+
+
+# ---------------------------------------------------------------- window split
+def test_split_window():
+    assert O.split_window(27) == (27, 13)
+    assert O.split_window(15) == (15, 7)
+    assert O.split_window(7) == (7, 3)
+    assert O.split_window(8) == (8, 3)          # even: left = W-1-W//2
+    assert O.split_window(1) == (1, 0)
+    assert O.split_window([9, 0]) == (9, 0)
+    assert O.split_window([9, 8]) == (9, 8)
+    for bad in (0, 81, [5, 5], [5, -1]):
+        with pytest.raises(ValueError):
+            O.split_window(bad)
+
+
+# ---------------------------------------------------------------- mask + softmax
+@pytest.mark.parametrize("T,W,L", GEOMS)
+def test_mask_closed_form(T, W, L):
+    pads = [0, 1, T // 2, T]
+    m = O.attn_mask(T, W, L, torch.tensor(pads))
+    assert m.shape == (len(pads), T, W)
+    for n, pad in enumerate(pads):
+        tv = T - pad
+        for t in range(T):
+            for j in range(W):
+                u = t - L + j
+                want = -100.0 if (t >= tv or u < 0 or u >= tv) else 0.0
+                assert m[n, t, j].item() == want
+    assert set(m.unique().tolist()) <= {0.0, -100.0}
+
+
+def test_zero_query_gives_softmax_of_bias_over_valid_slots():
+    N, H, T, W, L, C = 2, 3, 8, 5, 2, 8
+    rpb = _rand(H, W)
+    pad = torch.tensor([0, 3])
+    q = torch.zeros(N * H, T, C, dtype=F64)
+    k, v = _rand(N * H, T, C), _rand(N * H, T, C)
+    _, p, lse = O.na1d_forward(q, k, v, W, L, rpb, pad, H)
+    p = p.view(N, H, T, W)
+    for n in range(N):
+        tv = T - int(pad[n])
+        for h in range(H):
+            for t in range(T):
+                valid = [j for j in range(W) if 0 <= t - L + j < tv] if t < tv else []
+                if valid:
+                    want = torch.softmax(rpb[h, valid], 0)
+                    assert torch.allclose(p[n, h, t, valid], want, atol=1e-12)
+                    rest = [j for j in range(W) if j not in valid]
+                    assert (p[n, h, t, rest] < 1e-40).all()
+                else:  # fully padded row: uniform -100 shift cancels
+                    assert torch.allclose(p[n, h, t], torch.softmax(rpb[h], 0), atol=1e-12)
+    assert torch.allclose(p.sum(-1), torch.ones(N, H, T, dtype=F64), atol=1e-12)
+    z = O.logits(q, k, W, L, rpb, pad, H)
+    assert torch.allclose(lse, torch.log(torch.exp(z).sum(-1)), atol=1e-12)
+
+
+def test_interior_rows_equal_dense_local_softmax():
+    T, W, L, C = 12, 5, 2, 8
+    q, k, v = _rand(1, T, C), _rand(1, T, C), _rand(1, T, C)
+    o, _, _ = O.na1d_forward(q, k, v, W, L)
+    dense = (q @ k.transpose(1, 2))[0]
+    for t in range(T):
+        lo, hi = max(0, t - L), min(T, t + (W - 1 - L) + 1)
+        w = torch.softmax(dense[t, lo:hi], 0)
+        assert torch.allclose(o[0, t], w @ v[0, lo:hi], atol=1e-12)
+
+
+def test_padded_keys_do_not_reach_valid_rows():
+    N, H, T, W, L, C = 2, 2, 10, 5, 2, 8
+    pad = torch.tensor([4, 0])
+    q, k, v = _rand(N * H, T, C), _rand(N * H, T, C), _rand(N * H, T, C)
+    o1, _, _ = O.na1d_forward(q, k, v, W, L, None, pad, H)
+    k2, v2 = k.clone(), v.clone()
+    k2[:H, T - 4:] = 7.0
+    v2[:H, T - 4:] = -3.0
+    o2, _, _ = O.na1d_forward(q, k2, v2, W, L, None, pad, H)
+    assert torch.allclose(o1[:H, :T - 4], o2[:H, :T - 4], atol=1e-30)
+    assert torch.equal(o1[H:], o2[H:])
+
+
+# ---------------------------------------------------------------- gradients
+def test_gradcheck_fp64():
+    N, H, T, W, L, C = 1, 2, 6, 4, 1, 8
+    q, k, v = (_rand(N * H, T, C).requires_grad_(True) for _ in range(3))
+    rpb = _rand(H, W).requires_grad_(True)
+    pad = torch.tensor([1])
+    f = lambda q, k, v, r: O.na1d_forward(q, k, v, W, L, r, pad, H)[0]
+    assert torch.autograd.gradcheck(f, (q, k, v, rpb), eps=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("T,W,L", [(9, 5, 2), (3, 7, 3), (9, 4, 1), (12, 8, 3)])
+def test_formula_backward_equals_autograd(T, W, L):
+    N, H, C = 2, 2, 8
+    q, k, v, do = _rand(N * H, T, C), _rand(N * H, T, C), _rand(N * H, T, C), _rand(N * H, T, C)
+    rpb = _rand(H, W)
+    pad = torch.tensor([0, min(2, T)])
+    a = O.na1d_backward(q, k, v, do, W, L, rpb, pad, H)
+    b = O.na1d_backward_formulas(q, k, v, do, W, L, rpb, pad, H)
+    for x, y in zip(a, b):
+        assert torch.allclose(x, y, atol=1e-10)
+
+
+def test_batch_invariance():
+    """The reference's own (commented-out) smoke check: sample 0 alone equals
+    sample 0 inside a batch (pcf_nat_pytorch2.7.zip!/extension_na/test.py:24-51)."""
+    T, W, L, C = 20, 7, 3, 16
+    q, k, v = _rand(8, T, C), _rand(8, T, C), _rand(8, T, C)
+    o_all, _, _ = O.na1d_forward(q, k, v, W, L)
+    o_one, _, _ = O.na1d_forward(q[:1], k[:1], v[:1], W, L)
+    assert torch.allclose(o_all[:1], o_one, atol=1e-14)
+
+
+def test_seeded_inputs_are_reproducible_and_rounded():
+    a = O.seeded_qkv(2, 5, 8, seed=3, dtype=torch.bfloat16, scale_q=0.125)
+    b = O.seeded_qkv(2, 5, 8, seed=3, dtype=torch.bfloat16, scale_q=0.125)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    assert a[0].dtype == torch.bfloat16
+    assert math.isclose(O.rel_l2(a[1].float(), a[1].float()), 0.0)
