@@ -1,0 +1,200 @@
+#!/usr/bin/env python3
+"""NA1D benchmark on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input that is
+already resident in HBM: the fused NA1D forward followed by the fused backward
+(forward only for the forward-only workload), called through the C ABI on
+torch's current stream.  Inputs rotate over enough buffer sets to exceed the
+256 MB Infinity Cache, so cache hits do not pose as HBM bandwidth.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2]
+
+prints ONE JSON line.  `value` is algorithmic bytes per step / seconds per step
+(GB/s): 8*C bytes per token forward, 14*C backward (q,k,v[,dO] read and
+O / dQ,dK,dV written once, 16-bit; per-row statistics excluded).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "pcf-nat_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBPS = 8000.0
+
+# name: (N, H, T, C, W, dtype, backward?)   [B = N*H]
+WORKLOADS = {
+    "cfg1": dict(N=32, H=4, T=200, C=64, W=7, dtype="bf16", bwd=False,
+                 desc="NA1D fwd bf16 batch=32 heads=4 T=200 head_dim=64 window=7"),
+    "cfg2": dict(N=128, H=8, T=300, C=32, W=15, dtype="fp16", bwd=True,
+                 desc="NA1D fwd+bwd fp16 batch=128 heads=8 T=300 head_dim=32 window=15"),
+    "cfg3": dict(N=256, H=16, T=100, C=16, W=27, dtype="bf16", bwd=False,
+                 desc="NA layer of PCF-NAT 4x4 inference: batch=256 heads=16 T=100 head_dim=16 window=27, fwd bf16"),
+    "cfg4": dict(N=64, H=16, T=1000, C=16, W=27, dtype="bf16", bwd=False,
+                 desc="NA layer of PCF-NAT 6x4 at max length: batch=64 heads=16 T=1000 head_dim=16 window=27, fwd bf16"),
+    "cfg5": dict(N=128, H=16, T=100, C=16, W=27, dtype="fp16", bwd=True,
+                 desc="NA layer of MFA-NAT 4x4 training: batch=128 heads=16 T=100 head_dim=16 window=27, fwd+bwd fp16"),
+}
+
+# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# runs (see profiles/); None until measured for that workload.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(w):
+    tokens = w["N"] * w["H"] * w["T"]
+    fwd = 8 * w["C"] * tokens
+    bwd = 14 * w["C"] * tokens if w["bwd"] else 0
+    return fwd, bwd
+
+
+def make_sets(w, n_sets, device):
+    import torch
+    dt = torch.bfloat16 if w["dtype"] == "bf16" else torch.float16
+    B, T, C = w["N"] * w["H"], w["T"], w["C"]
+    g = torch.Generator(device="cpu").manual_seed(0)
+    sets = []
+    for _ in range(n_sets):
+        s = {}
+        for name in ("q", "k", "v", "do"):
+            s[name] = torch.randn(B, T, C, generator=g, dtype=torch.float32).to(dt).to(device)
+        s["q"] = s["q"] * (C ** -0.5)
+        s["rpb"] = (torch.randn(w["H"], w["W"], generator=g) * 0.02).to(device)
+        s["o"] = torch.empty_like(s["q"])
+        s["lse"] = torch.empty(B, T, dtype=torch.float32, device=device)
+        if w["bwd"]:
+            for name in ("dq", "dk", "dv"):
+                s[name] = torch.empty_like(s["q"])
+            s["drpb"] = torch.zeros(w["H"], w["W"], dtype=torch.float32, device=device)
+        sets.append(s)
+    return sets
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """The oracle (CPU restatement of the reference math, PyTorch fp32) timed on
+    this host's cores on a bounded sample of the same workload."""
+    import torch
+    from oracle import na1d_oracle as O
+    cores = os.cpu_count() or 1
+    threads = min(cores, 16)
+    torch.set_num_threads(threads)
+    H, T, C, W = w["H"], w["T"], w["C"], w["W"]
+    _, L = O.split_window(W)
+    n_sample = max(1, min(w["N"], 16))
+    B = n_sample * H
+    q, k, v, do = O.seeded_qkv(B, T, C, seed=0, dtype=torch.float32, n=4)
+    rpb = torch.zeros(H, W)
+
+    def run():
+        if w["bwd"]:
+            O.na1d_forward(q, k, v, W, L, rpb, None, H)
+            O.na1d_backward_formulas(q, k, v, do, W, L, rpb, None, H)
+        else:
+            O.na1d_forward(q, k, v, W, L, rpb, None, H)
+
+    run()
+    times, t_start = [], time.perf_counter()
+    while len(times) < 5 or (time.perf_counter() - t_start < budget_s / 2 and len(times) < 30):
+        t0 = time.perf_counter()
+        run()
+        times.append(time.perf_counter() - t0)
+    sec = statistics.median(times)
+    fwd_b, bwd_b = algorithmic_bytes(dict(w, N=n_sample))
+    return {"value": (fwd_b + bwd_b) / sec / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "%d of %d samples (B=%d rows of T=%d), median of %d runs, %.3f s each, PyTorch CPU fp32"
+                      % (n_sample, w["N"], B, T, len(times), sec)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the op shards over "
+              "batch*heads with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from na1d_amd import _lib
+    from oracle import na1d_oracle as O
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _lib.load()
+    dev = torch.device("cuda:0")
+    w = WORKLOADS[args.workload]
+    H, T, C, W = w["H"], w["T"], w["C"], w["W"]
+    B = w["N"] * H
+    _, L = O.split_window(W)
+    fwd_bytes, bwd_bytes = algorithmic_bytes(w)
+    set_bytes = fwd_bytes + bwd_bytes
+    n_sets = max(2, int(600e6 // set_bytes) + 1)      # > 2x the 256 MB Infinity Cache in rotation
+    sets = make_sets(w, n_sets, dev)
+
+    def fwd(s):
+        _lib.call_fused_forward(s["o"], s["lse"], s["q"], s["k"], s["v"], s["rpb"], None, B, H, T, C, W, L, 1.0)
+
+    def bwd(s):
+        _lib.call_fused_backward(s["dq"], s["dk"], s["dv"], s["drpb"], s["q"], s["k"], s["v"], s["o"], s["do"],
+                                 s["lse"], s["rpb"], None, B, H, T, C, W, L, 1.0)
+
+    for i in range(max(args.warmup, 1)):
+        s = sets[i % n_sets]
+        fwd(s)
+        if w["bwd"]:
+            bwd(s)
+    torch.cuda.synchronize()
+
+    # timed region: exactly K steps, whole-step wall clock + per-kernel HIP events
+    K = args.steps
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(K)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(K):
+        s = sets[i % n_sets]
+        ev[i][0].record()
+        fwd(s)
+        ev[i][1].record()
+        if w["bwd"]:
+            bwd(s)
+            ev[i][2].record()
+    torch.cuda.synchronize()
+    sec = time.perf_counter() - t0
+    ms_per_step = sec / K * 1e3
+    fwd_ms = statistics.mean(e[0].elapsed_time(e[1]) for e in ev)
+    bwd_ms = statistics.mean(e[1].elapsed_time(e[2]) for e in ev) if w["bwd"] else None
+
+    value = set_bytes / (sec / K) / 1e9
+    if w["bwd"]:
+        dom_name, dom_bytes, dom_ms = "fused backward", bwd_bytes, bwd_ms
+    else:
+        dom_name, dom_bytes, dom_ms = "fused forward", fwd_bytes, fwd_ms
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    line = {
+        "metric": "NA1D fwd+bwd HBM GB/s (% of peak); PCF-NAT 4x4 embeddings/sec on 1 MI355X",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": w["desc"], "name": args.workload, "B": B, "T": T, "C": C, "W": W, "left": L,
+                   "buffer_sets_rotated": n_sets, "algorithmic_bytes_per_step": set_bytes,
+                   "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "kernel": dom_name, "kernel_ms": round(dom_ms, 5), "algorithmic_bytes": dom_bytes},
+        "kernels_ms": {"fused_forward": round(fwd_ms, 5), "fused_backward": None if bwd_ms is None else round(bwd_ms, 5)},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

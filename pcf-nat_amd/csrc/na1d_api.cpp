@@ -1,5 +1,7 @@
 // C ABI of libna1d: argument validation and dispatch.  No torch types, no
 // allocation, no global mutable state; kernels go to the stream that is passed in.
+#include <cstdlib>
+
 #include "na1d_common.h"
 
 namespace {
@@ -37,16 +39,23 @@ int check(const void *o, const void *a, const void *b, int64_t B, int64_t T, int
         if (st != NA1D_OK) return st > 0 ? NA1D_OK : st; \
     }
 
+// NA1D_FORCE_GENERIC=1 in the environment routes every call to the generic
+// kernels (a second, independent implementation; used by the tests to cross-check).
+inline bool mfma_allowed() {
+    const char *e = std::getenv("NA1D_FORCE_GENERIC");
+    return !(e && e[0] == '1');
+}
+
 int band_qk(void *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s) {
-    const int st = na1d::mfma::qk((float *)attn, a, b, g, dtype, s);
+    const int st = mfma_allowed() ? na1d::mfma::qk((float *)attn, a, b, g, dtype, s) : NA1D_ERR_UNSUPPORTED;
     return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::qk((float *)attn, a, b, g, dtype, s) : st;
 }
 int band_av(void *out, const void *attn, const void *v, const Geom &g, int dtype, hipStream_t s) {
-    const int st = na1d::mfma::av(out, (const float *)attn, v, g, dtype, s);
+    const int st = mfma_allowed() ? na1d::mfma::av(out, (const float *)attn, v, g, dtype, s) : NA1D_ERR_UNSUPPORTED;
     return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::av(out, (const float *)attn, v, g, dtype, s) : st;
 }
 int band_gather(void *out, const void *attn, const void *x, const Geom &g, int dtype, hipStream_t s) {
-    const int st = na1d::mfma::gather(out, (const float *)attn, x, g, dtype, s);
+    const int st = mfma_allowed() ? na1d::mfma::gather(out, (const float *)attn, x, g, dtype, s) : NA1D_ERR_UNSUPPORTED;
     return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::gather(out, (const float *)attn, x, g, dtype, s) : st;
 }
 
@@ -113,7 +122,9 @@ int na1d_fused_forward(void *out, float *lse, const void *q, const void *k, cons
     NA1D_CHECK(out, q, k, B, T, C, W, left, H, dtype, g);
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
-    const int st = na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream);
+    const int st = mfma_allowed()
+                       ? na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream)
+                       : NA1D_ERR_UNSUPPORTED;
     if (st != NA1D_ERR_UNSUPPORTED) return st;
     return na1d::generic::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream);
 }
@@ -126,8 +137,9 @@ int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb, const void *q
     if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
         return NA1D_ERR_ALIGN;
-    const int st = na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, scale, dtype,
-                                         (hipStream_t)stream);
+    const int st = mfma_allowed() ? na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g,
+                                                          scale, dtype, (hipStream_t)stream)
+                                  : NA1D_ERR_UNSUPPORTED;
     if (st != NA1D_ERR_UNSUPPORTED) return st;
     return na1d::generic::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, scale, dtype,
                                     (hipStream_t)stream);

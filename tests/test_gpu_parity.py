@@ -26,6 +26,13 @@ SHAPES = [
 ]
 
 
+def _err(got, ref):
+    """rel-L2, with an absolute floor so that references that are zero up to
+    e^-100 (e.g. d rpb of a one-token sequence) do not divide by nothing."""
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    return (got - ref).norm().item() / max(ref.norm().item(), 1e-6)
+
+
 def _unfused(name, out, a, b, W, left):
     B, T, C = (a if a.dtype != torch.float32 else b).shape
     _lib.call_unfused(name, out, a, b, B, T, C, W, left, (a if a.dtype != torch.float32 else b).dtype)
@@ -120,7 +127,7 @@ def test_dropin_autograd_chain_matches_oracle(geom, dtype):
     assert O.rel_l2(qd.grad.float(), wq) < tol
     assert O.rel_l2(kd.grad.float(), wk) < tol
     assert O.rel_l2(vd.grad.float(), wv) < tol
-    assert O.rel_l2(rd.grad, wr) < tol
+    assert _err(rd.grad, wr) < tol
 
 
 FUSED_GEOMS = [  # (N, H, T, C, W, left)
@@ -155,7 +162,7 @@ def test_fused_forward_backward_matches_oracle(geom, dtype):
     assert O.rel_l2(qd.grad.float(), wq) < tol, "dQ"
     assert O.rel_l2(kd.grad.float(), wk) < tol, "dK"
     assert O.rel_l2(vd.grad.float(), wv) < tol, "dV"
-    assert O.rel_l2(rd.grad, wr) < tol, "drpb"
+    assert _err(rd.grad, wr) < tol, "drpb"
     _, lse = na1d_fused_forward_lse(qd.detach(), kd.detach(), vd.detach(), W, L, rd.detach(), t_valid.cuda(), H)
     assert torch.allclose(lse.cpu(), want_lse, atol=2e-3, rtol=1e-4), "LSE"
 
