@@ -52,7 +52,10 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define LDS_PTR(T) __attribute__((address_space(3))) T *
 
-constexpr int kWaves = 4;            // waves per workgroup
+#ifndef NA1D_WAVES
+#define NA1D_WAVES 4
+#endif
+constexpr int kWaves = NA1D_WAVES;   // waves per workgroup
 constexpr int kThreads = 64 * kWaves;
 constexpr float kNegInf = -__builtin_inff();
 
@@ -217,25 +220,29 @@ template <int NBV> struct Window {
     u32x2 keep0, keep2;           // NBV 3: 16-bit lane masks that split packed X into blocks 0 and 2
 };
 
+// `bias_lds` holds this head's rpb row times log2(e) in slots [0, W) (zeros without
+// rpb); it is filled by stage_bias() before the workgroup barrier.
+__device__ inline void stage_bias(LDS_PTR(float) bias_lds, const float *rpb_h, int W, int tid) {
+    if (tid < 32) bias_lds[tid] = (rpb_h && tid < W) ? rpb_h[tid] * kLog2e : 0.f;
+}
+__device__ inline float bias_at(LDS_PTR(float) bias_lds, int j, int W) {   // -inf outside the band
+    const float val = bias_lds[j & 31];
+    return (j >= 0 && j < W) ? val : kNegInf;
+}
+
 template <int NBV>
-__device__ inline void make_window(Window<NBV> &w, const float *rpb_h, int W, int L, int shift, int g, int n) {
-    const Rsrc rb = make_rsrc(rpb_h, rpb_h ? W * 4 : 0);
-    auto rpb_at = [&](int j) {   // rpb[j]*log2e inside the band, -inf outside
-        const float val = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rb, j * 4, 0, 0));   // 0 outside [0,W)
-        return (j >= 0 && j < W) ? val * kLog2e : kNegInf;
-    };
+__device__ inline void make_window(Window<NBV> &w, LDS_PTR(float) bias_lds, int W, int L, int shift, int g, int n) {
     uint32_t m[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int j0 = 4 * g + r - shift - n + L;
-        w.bias_y[r] = rpb_at(j0 + 16);
+        w.bias_y[r] = bias_at(bias_lds, j0 + 16, W);
         if (NBV == 2) {
             w.from0[r] = true;
-            w.bias_x[r] = rpb_at(j0);
+            w.bias_x[r] = bias_at(bias_lds, j0, W);
         } else {
             w.from0[r] = j0 >= 0;
-            const float b0 = rpb_at(j0), b2 = rpb_at(j0 + 32);
-            w.bias_x[r] = w.from0[r] ? b0 : b2;
+            w.bias_x[r] = bias_at(bias_lds, w.from0[r] ? j0 : j0 + 32, W);
         }
         m[r] = w.from0[r] ? 0xffffu : 0u;
     }
@@ -285,9 +292,11 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     constexpr int MT = Strip<C>::kMaxTiles;
     constexpr int kKeyRegion = (MT + 2) * LL::kTileBytes;
     __shared__ __attribute__((aligned(16))) char smem[2 * kKeyRegion + MT * LL::kTileBytes];
+    __shared__ float bias_smem[32];
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + kKeyRegion;
     LDS_PTR(char) q_lds = v_lds + kKeyRegion;
+    LDS_PTR(float) bias_lds = (LDS_PTR(float))bias_smem;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -315,6 +324,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         sk.issue(ks, 16 * i0 - 16, tid);
         sv.issue(vs, 16 * i0 - 16, tid);
         sq.issue(qs, 16 * i0, tid);
+        stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
         sk.commit(k_lds, tid);
         sv.commit(v_lds, tid);
         sq.commit(q_lds, tid);
@@ -322,8 +332,6 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
-    Window<NBV> win;
-    make_window<NBV>(win, rpb ? rpb + head * W : nullptr, W, L, shift, g, n);
     const float scale2 = scale * kLog2e;
 
     // per-lane LDS offsets; key-side regions start 16 rows before the strip
@@ -334,6 +342,8 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     v_lane.init(16 - shift, lane);
 
     __syncthreads();
+    Window<NBV> win;
+    make_window<NBV>(win, bias_lds, W, L, shift, g, n);
 
     for (int i = i0 + wave; i < i1; i += kWaves) {
         const int tile_bytes = (i - i0) * LL::kTileBytes;
@@ -500,7 +510,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     constexpr int kQryRegion = (MT + 2) * LL::kTileBytes;    // rows 16*i0 - 16 ...
     constexpr int kRowsQ = (MT + 2) * 16;
     __shared__ __attribute__((aligned(16))) char smem[2 * kKeyRegion + 2 * kQryRegion];
-    __shared__ __attribute__((aligned(16))) float lse_lds[kRowsQ], delta_lds[kRowsQ], drpb_lds[32];
+    __shared__ __attribute__((aligned(16))) float lse_lds[kRowsQ], delta_lds[kRowsQ], drpb_lds[32], bias_smem[32];
+    LDS_PTR(float) bias_lds = (LDS_PTR(float))bias_smem;
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + kKeyRegion;
     LDS_PTR(char) q_lds = v_lds + kKeyRegion;
@@ -531,6 +542,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         sg.issue(gs, 16 * i0 - 16, tid);
         float l = 0.f;
         if (tid < kRowsQ) l = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ls, (16 * i0 - 16 + tid) * 4, 0, 0));
+        stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
         sk.commit(k_lds, tid);
         sv.commit(v_lds, tid);
         sq.commit(q_lds, tid);
@@ -541,9 +553,6 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
-    const float *rpb_h = rpb ? rpb + head * W : nullptr;
-    Window<NBV> win;
-    make_window<NBV>(win, rpb_h, W, L, shift, g, n);
     const float scale2 = scale * kLog2e;
     const float mask2 = kMaskValue * kLog2e;
 
@@ -555,6 +564,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     qry_tr.init(0, lane);
 
     __syncthreads();
+    Window<NBV> win;
+    make_window<NBV>(win, bias_lds, W, L, shift, g, n);
 
     // ---------------- pass 1: query tiles i0-1 .. i1 -> delta, dQ, drpb ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
@@ -663,17 +674,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
     // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb
     float bias2[NBV][4];
-    {
-        const Rsrc rb = make_rsrc(rpb_h, rpb_h ? W * 4 : 0);
 #pragma unroll
-        for (int vb = 0; vb < NBV; ++vb)
+    for (int vb = 0; vb < NBV; ++vb)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int j = 16 * vb - shift + n - (4 * g + r) + L;
-                const float val = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rb, j * 4, 0, 0));
-                bias2[vb][r] = (j >= 0 && j < W) ? val * kLog2e : kNegInf;
-            }
-    }
+        for (int r = 0; r < 4; ++r) bias2[vb][r] = bias_at(bias_lds, 16 * vb - shift + n - (4 * g + r) + L, W);
     const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
     const Rsrc dks = make_rsrc(dk + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
     const Rsrc dvs = make_rsrc(dv + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
