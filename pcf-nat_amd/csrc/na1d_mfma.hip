@@ -199,11 +199,23 @@ __device__ inline void swap_rows32(float x, float &a, float &b) {
     a = __uint_as_float(r.x);
     b = __uint_as_float(r.y);
 }
+// Plain v_max_f32 / v_max3_f32: scores are never NaN, so the quieting that fmaxf()
+// adds in front of every operand is skipped.
+__device__ inline float max2(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ inline float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 __device__ inline float xor_max(float x) {
     float a, b;
     swap_rows16(x, a, b);
-    swap_rows32(fmaxf(a, b), a, b);
-    return fmaxf(a, b);
+    swap_rows32(max2(a, b), a, b);
+    return max2(a, b);
 }
 __device__ inline float xor_sum(float x) {
     float a, b;
@@ -369,19 +381,18 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         // additive -100 of the model's mask, only on tiles that touch an edge
         const int s0 = 16 * i - shift;           // first row of the window
         const int qrow = 16 * i + n;
-        float lse_shift = 0.f;
         if (s0 < 0 || s0 + 16 * NBV > tv) {
-            if (qrow >= tv) lse_shift = kMaskValue;          // whole row shifted: softmax unchanged
+            const bool row_masked = qrow >= tv;  // a padded query row masks all of its slots
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int key_y = s0 + 16 + 4 * g + r;
-                const int key_x = s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0);
-                zx[r] += ((key_x < 0 || key_x >= tv) && qrow < tv) ? kMaskValue * kLog2e : 0.f;
-                zy[r] += ((key_y < 0 || key_y >= tv) && qrow < tv) ? kMaskValue * kLog2e : 0.f;
+                const uint32_t key_y = (uint32_t)(s0 + 16 + 4 * g + r);
+                const uint32_t key_x = (uint32_t)(s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0));
+                zx[r] += (key_x >= (uint32_t)tv || row_masked) ? kMaskValue * kLog2e : 0.f;   // unsigned: also key < 0
+                zy[r] += (key_y >= (uint32_t)tv || row_masked) ? kMaskValue * kLog2e : 0.f;
             }
         }
 
-        float m = fmaxf(fmaxf(fmaxf(zx[0], zx[1]), fmaxf(zx[2], zx[3])), fmaxf(fmaxf(zy[0], zy[1]), fmaxf(zy[2], zy[3])));
+        float m = max3(max3(zx[0], zx[1], zx[2]), max3(zx[3], zy[0], zy[1]), max2(zy[2], zy[3]));
         m = xor_max(m);
 
         float px[4], py[4], sum = 0.f;
@@ -425,7 +436,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         }
         if (g == 0)
             __builtin_amdgcn_raw_buffer_store_b32(
-                __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2 + lse_shift), ls, qrow * 4, 0, 0);
+                __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2), ls, qrow * 4, 0, 0);
     }
 }
 
@@ -604,10 +615,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         if (s0 < 0 || s0 + 16 * NBV > tv) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const int key_y = s0 + 16 + 4 * g + r;
-                const int key_x = s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0);
-                zx[r] += (key_x < 0 || key_x >= tv || qrow >= tv) ? mask2 : 0.f;
-                zy[r] += (key_y < 0 || key_y >= tv || qrow >= tv) ? mask2 : 0.f;
+                const uint32_t key_y = (uint32_t)(s0 + 16 + 4 * g + r);
+                const uint32_t key_x = (uint32_t)(s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0));
+                zx[r] += (key_x >= (uint32_t)tv || qrow >= tv) ? mask2 : 0.f;   // unsigned: also key < 0
+                zy[r] += (key_y >= (uint32_t)tv || qrow >= tv) ? mask2 : 0.f;
             }
         }
         float px[4], py[4], part = 0.f;
@@ -710,7 +721,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int qrow = 16 * qt + 4 * g + r;
-                    z[r] += (key < 0 || key >= tv || qrow >= tv) ? mask2 : 0.f;
+                    z[r] += ((uint32_t)key >= (uint32_t)tv || qrow >= tv) ? mask2 : 0.f;
                 }
             }
             float pp[4], ds[4];
