@@ -114,13 +114,24 @@ int na1d_fused_forward(void *out, float *lse,
  * (it already includes `scale`).
  *
  *   drpb : fp32 [H, W], ACCUMULATED into (caller zeroes it), or NULL to skip
+ *   workspace, workspace_bytes : optional device scratch for the d rpb reduction.
+ *          With at least na1d_fused_backward_workspace_bytes(...) bytes the per-
+ *          workgroup partial sums go there and a second small kernel folds them in a
+ *          fixed order; with NULL / too few bytes they are added with float atomics
+ *          (slower under contention, order not reproducible).  Contents need no
+ *          initialisation and are not meaningful afterwards.
  */
 int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb,
                         const void *q, const void *k, const void *v,
                         const void *out, const void *dout, const float *lse,
                         const float *rpb, const int32_t *t_valid,
                         int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
-                        float scale, int dtype, void *stream);
+                        float scale, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+
+/* Bytes of workspace na1d_fused_backward can use for these arguments (0 if it has
+ * no use for one, negative status on invalid arguments). */
+int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
+                                            int dtype);
 
 #ifdef __cplusplus
 }

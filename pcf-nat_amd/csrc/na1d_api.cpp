@@ -10,10 +10,9 @@ using na1d::Geom;
 
 inline bool misaligned(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
 
-// Common checks of the un-fused entry points.  Returns NA1D_OK, an error, or
-// +1 for "nothing to do".
-int check(const void *o, const void *a, const void *b, int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
-          int64_t H, int dtype, Geom &g) {
+// Shape checks shared by every entry point.  Returns NA1D_OK, an error, or +1 for
+// "nothing to do".
+int check_shape(int64_t B, int64_t T, int64_t C, int64_t W, int64_t left, int64_t H, int dtype, Geom &g) {
     if (dtype != NA1D_BF16 && dtype != NA1D_FP16) return NA1D_ERR_DTYPE;
     if (C <= 0 || C % 8 != 0 || C > (1 << 20)) return NA1D_ERR_HEAD_DIM;
     if (W < 1 || W > NA1D_MAX_WINDOW || left < 0 || left >= W) return NA1D_ERR_WINDOW;
@@ -21,14 +20,22 @@ int check(const void *o, const void *a, const void *b, int64_t B, int64_t T, int
     if (B == 0 || T == 0) return 1;
     const int64_t widest = C > W ? C : W;
     if (T > (INT64_MAX / 8) / widest || B > (INT64_MAX / 8) / (T * widest)) return NA1D_ERR_SHAPE;
-    if (!o || !a || !b) return NA1D_ERR_NULL;
-    if (misaligned(o) || misaligned(a) || misaligned(b)) return NA1D_ERR_ALIGN;
     g.B = B;
     g.T = T;
     g.C = (int)C;
     g.W = (int)W;
     g.L = (int)left;
     g.H = (int)H;
+    return NA1D_OK;
+}
+
+// Shape checks plus the three pointers every entry point has.
+int check(const void *o, const void *a, const void *b, int64_t B, int64_t T, int64_t C, int64_t W, int64_t left,
+          int64_t H, int dtype, Geom &g) {
+    const int st = check_shape(B, T, C, W, left, H, dtype, g);
+    if (st != NA1D_OK) return st;
+    if (!o || !a || !b) return NA1D_ERR_NULL;
+    if (misaligned(o) || misaligned(a) || misaligned(b)) return NA1D_ERR_ALIGN;
     return NA1D_OK;
 }
 
@@ -132,17 +139,29 @@ int na1d_fused_forward(void *out, float *lse, const void *q, const void *k, cons
 int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
                         const void *out, const void *dout, const float *lse, const float *rpb,
                         const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
-                        int64_t left, float scale, int dtype, void *stream) {
+                        int64_t left, float scale, int dtype, void *workspace, int64_t workspace_bytes,
+                        void *stream) {
     NA1D_CHECK(dq, q, k, B, T, C, W, left, H, dtype, g);
     if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
         return NA1D_ERR_ALIGN;
+    if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
     const int st = mfma_allowed() ? na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g,
-                                                          scale, dtype, (hipStream_t)stream)
+                                                          scale, dtype, (float *)workspace,
+                                                          workspace ? workspace_bytes : 0, (hipStream_t)stream)
                                   : NA1D_ERR_UNSUPPORTED;
     if (st != NA1D_ERR_UNSUPPORTED) return st;
     return na1d::generic::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, scale, dtype,
-                                    (hipStream_t)stream);
+                                    (hipStream_t)stream);   // the generic kernel has no use for the workspace
+}
+
+int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
+                                            int dtype) {
+    Geom g;
+    const int st = check_shape(B, T, C, W, left, H, dtype, g);
+    if (st < 0) return st;
+    if (st > 0 || !mfma_allowed()) return 0;
+    return na1d::mfma::fused_bwd_workspace_bytes(g, dtype);
 }
 
 }  // extern "C"

@@ -98,7 +98,9 @@ int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v
               const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s);
 int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
               const void *out, const void *dout, const float *lse, const float *rpb,
-              const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s);
+              const int32_t *t_valid, const Geom &g, float scale, int dtype, float *workspace,
+              int64_t workspace_bytes, hipStream_t s);
+int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype);   // 0 when the shape is not covered
 }  // namespace mfma
 
 }  // namespace na1d

@@ -115,9 +115,11 @@ template <int C> struct Strip {
     static constexpr int kMaxTiles = C <= 16 ? 8 : C <= 32 ? 8 : C <= 64 ? 4 : 2;
 };
 
-// Copy rows [row_lo, row_lo + 16*NTILES) of a sequence into an LDS region, all loads in
-// flight before the first LDS store.  Split in two so several regions' loads can be
-// issued back to back.
+// Copy up to NTILES tiles of rows, starting at row_lo of a sequence, into an LDS
+// region, all loads in flight before the first LDS store.  Split in two so several
+// regions' loads can be issued back to back.  NTILES fixes the (unrolled) number of
+// loads per thread; the caller's buffer resource ends where the wanted rows end, so
+// surplus loads fetch nothing.
 template <int C, int NTILES> struct Stage {
     static constexpr int kTotal = NTILES * 16 * Lds<C>::kUnits;             // 16-byte units
     static constexpr int kRounds = (kTotal + kThreads - 1) / kThreads;
@@ -127,11 +129,13 @@ template <int C, int NTILES> struct Stage {
         for (int j = 0; j < kRounds; ++j)
             x[j] = __builtin_amdgcn_raw_buffer_load_b128(src, (row_lo * Lds<C>::kUnits + j * kThreads + tid) * 16, 0, 0);
     }
-    __device__ inline void commit(LDS_PTR(char) region, int tid) const {
+    // `ntiles` <= NTILES: the region only has room for that many tiles
+    __device__ inline void commit(LDS_PTR(char) region, int ntiles, int tid) const {
+        const int total = ntiles * 16 * Lds<C>::kUnits;
 #pragma unroll
         for (int j = 0; j < kRounds; ++j) {
             const int u = j * kThreads + tid;
-            if (kTotal % kThreads == 0 || u < kTotal)
+            if (u < total)
                 *reinterpret_cast<LDS_PTR(u32x4)>(region + Lds<C>::addr(u / Lds<C>::kUnits, (u % Lds<C>::kUnits) * 16)) = x[j];
         }
     }
@@ -302,13 +306,13 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     using LL = Lds<C>;
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = Strip<C>::kMaxTiles;
-    constexpr int kKeyRegion = (MT + 2) * LL::kTileBytes;
-    __shared__ __attribute__((aligned(16))) char smem[2 * kKeyRegion + MT * LL::kTileBytes];
-    __shared__ float bias_smem[32];
+    // dynamic LDS (fwd_lds_bytes): K and V regions of nt+2 tiles, Q region of nt tiles, 32 bias floats
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int key_region = (nt + 2) * LL::kTileBytes;
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) v_lds = k_lds + kKeyRegion;
-    LDS_PTR(char) q_lds = v_lds + kKeyRegion;
-    LDS_PTR(float) bias_lds = (LDS_PTR(float))bias_smem;
+    LDS_PTR(char) v_lds = k_lds + key_region;
+    LDS_PTR(char) q_lds = v_lds + key_region;
+    LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + nt * LL::kTileBytes);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -337,9 +341,9 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         sv.issue(vs, 16 * i0 - 16, tid);
         sq.issue(qs, 16 * i0, tid);
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
-        sk.commit(k_lds, tid);
-        sv.commit(v_lds, tid);
-        sq.commit(q_lds, tid);
+        sk.commit(k_lds, nt + 2, tid);
+        sv.commit(v_lds, nt + 2, tid);
+        sq.commit(q_lds, nt, tid);
     }
 
     int tv = T;
@@ -373,7 +377,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         float zx[4], zy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[2][r]) : s[0][r];
+            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[NBV - 1][r]) : s[0][r];
             zx[r] = __builtin_fmaf(sx, scale2, win.bias_x[r]);
             zy[r] = __builtin_fmaf(s[1][r], scale2, win.bias_y[r]);
         }
@@ -412,7 +416,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         pb[1] = pky;
         if (NBV == 3) {
             pb[0] = u32x2{pkx.x & win.keep0.x, pkx.y & win.keep0.y};
-            pb[2] = u32x2{pkx.x & win.keep2.x, pkx.y & win.keep2.y};
+            pb[NBV - 1] = u32x2{pkx.x & win.keep2.x, pkx.y & win.keep2.y};
         } else {
             pb[0] = pkx;
         }
@@ -440,6 +444,14 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     }
 }
 
+// Dynamic LDS above 64 KB has to be allowed per kernel.
+template <class K>
+inline bool allow_lds(K kern, size_t bytes) {
+    if (bytes <= 64 * 1024) return true;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)bytes) == hipSuccess;
+}
+
 // Number of virtual key blocks the kernels need, 0 if the shape is not covered.
 inline int window_blocks(const Geom &g) {
     const int R = g.W - 1 - g.L;
@@ -456,7 +468,9 @@ int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
     if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
     auto kern = window_blocks(g) == 2 ? fused_fwd_kernel<DT, C, 2> : fused_fwd_kernel<DT, C, 3>;
-    kern<<<(unsigned)sp.items, kThreads, 0, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
+    const size_t lds = (size_t)(3 * sp.nt + 4) * Lds<C>::kTileBytes + 32 * sizeof(float);
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                                                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
                                                  sp.nt, sp.strips, scale);
     return launch_status();
@@ -503,6 +517,29 @@ int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v
 //     atomics, each output row written once.
 // The score work is done twice so that both contractions find their B operand
 // already in accumulator layout and nothing is exchanged between waves.
+// d rpb partial sums: one row of kPartialStride floats per work item, folded in a
+// fixed order by a second kernel (one workgroup per head).
+constexpr int kPartialStride = 32;
+
+__global__ void __launch_bounds__(128)
+drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, int N, int H, int strips, int W) {
+    __shared__ float acc[128];
+    const int h = blockIdx.x / W, j = blockIdx.x - h * W;
+    const int rows = N * strips;                      // items of this head: (n, strip)
+    float s = 0.f;
+    for (int i = threadIdx.x; i < rows; i += 128) {
+        const int n = i / strips, st = i - n * strips;
+        s += partial[((size_t)(n * H + h) * strips + st) * kPartialStride + j];
+    }
+    acc[threadIdx.x] = s;
+    __syncthreads();
+    for (int half = 64; half > 0; half >>= 1) {       // fixed tree: the result does not depend on timing
+        if ((int)threadIdx.x < half) acc[threadIdx.x] += acc[threadIdx.x + half];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) drpb[h * W + j] += acc[0];
+}
+
 template <int C> struct StripBwd {
     static constexpr int kMaxTiles = C <= 32 ? 8 : C <= 64 ? 4 : 2;
 };
@@ -513,20 +550,26 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
-                 int strips, float scale) {
+                 int strips, float scale, float *__restrict__ drpb_partial) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
-    constexpr int kKeyRegion = (MT + 4) * LL::kTileBytes;    // rows 16*i0 - 32 ...
-    constexpr int kQryRegion = (MT + 2) * LL::kTileBytes;    // rows 16*i0 - 16 ...
     constexpr int kRowsQ = (MT + 2) * 16;
-    __shared__ __attribute__((aligned(16))) char smem[2 * kKeyRegion + 2 * kQryRegion];
-    __shared__ __attribute__((aligned(16))) float lse_lds[kRowsQ], delta_lds[kRowsQ], drpb_lds[32], bias_smem[32];
-    LDS_PTR(float) bias_lds = (LDS_PTR(float))bias_smem;
+    static_assert(kRowsQ <= kThreads, "one thread per staged lse row");
+    // dynamic LDS (bwd_lds_bytes): K, V regions of nt+4 tiles (rows 16*i0 - 32 ...), Q, dO regions of nt+2 tiles
+    // (rows 16*i0 - 16 ...), lse and delta of the query-side rows, 32 bias floats, and - only when d rpb is
+    // wanted - per-lane partial sums and 8 partial sums per slot
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int key_region = (nt + 4) * LL::kTileBytes, qry_region = (nt + 2) * LL::kTileBytes;
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) v_lds = k_lds + kKeyRegion;
-    LDS_PTR(char) q_lds = v_lds + kKeyRegion;
-    LDS_PTR(char) g_lds = q_lds + kQryRegion;      // dO
+    LDS_PTR(char) v_lds = k_lds + key_region;
+    LDS_PTR(char) q_lds = v_lds + key_region;
+    LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
+    LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
+    LDS_PTR(float) delta_lds = lse_lds + kRowsQ;
+    LDS_PTR(float) bias_lds = delta_lds + kRowsQ;
+    LDS_PTR(float) rpart = bias_lds + 32;          // [kWaves * 8][64]
+    LDS_PTR(float) rsum = rpart + kWaves * 8 * 64; // [8][32]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -554,12 +597,11 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         float l = 0.f;
         if (tid < kRowsQ) l = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ls, (16 * i0 - 16 + tid) * 4, 0, 0));
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
-        sk.commit(k_lds, tid);
-        sv.commit(v_lds, tid);
-        sq.commit(q_lds, tid);
-        sg.commit(g_lds, tid);
+        sk.commit(k_lds, nt + 4, tid);
+        sv.commit(v_lds, nt + 4, tid);
+        sq.commit(q_lds, nt + 2, tid);
+        sg.commit(g_lds, nt + 2, tid);
         if (tid < kRowsQ) lse_lds[tid] = l * kLog2e;
-        if (tid < 32) drpb_lds[tid] = 0.f;
     }
 
     int tv = T;
@@ -604,8 +646,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         float zx[4], zy[4], dpx[4], dpy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[2][r]) : s[0][r];
-            dpx[r] = NBV == 3 ? (win.from0[r] ? dp[0][r] : dp[2][r]) : dp[0][r];
+            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[NBV - 1][r]) : s[0][r];
+            dpx[r] = NBV == 3 ? (win.from0[r] ? dp[0][r] : dp[NBV - 1][r]) : dp[0][r];
             dpy[r] = dp[1][r];
             zx[r] = __builtin_fmaf(sx, scale2, win.bias_x[r]) - lse2;
             zy[r] = __builtin_fmaf(s[1][r], scale2, win.bias_y[r]) - lse2;
@@ -646,7 +688,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         db[1] = u32x2{Mma<DT>::pack(dsy[0], dsy[1]), Mma<DT>::pack(dsy[2], dsy[3])};
         if (NBV == 3) {
             db[0] = u32x2{pkx.x & win.keep0.x, pkx.y & win.keep0.y};
-            db[2] = u32x2{pkx.x & win.keep2.x, pkx.y & win.keep2.y};
+            db[NBV - 1] = u32x2{pkx.x & win.keep2.x, pkx.y & win.keep2.y};
         } else {
             db[0] = pkx;
         }
@@ -668,19 +710,35 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
 
-    // d rpb: slot j of this lane is fixed across tiles; fold lanes through LDS, one atomic per slot
+    // d rpb: the window slot of each of a lane's 8 score registers is the same for every tile, so the
+    // lane keeps running sums; they are folded across lanes and waves through LDS in a fixed order.
     if (drpb) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int j0 = 4 * g + r - shift - n + L;
-            const int jx = (NBV == 3 && !win.from0[r]) ? j0 + 32 : j0, jy = j0 + 16;
-            if (jx >= 0 && jx < W) atomicAdd(&drpb_lds[jx], racc_x[r]);
-            if (jy >= 0 && jy < W) atomicAdd(&drpb_lds[jy], racc_y[r]);
+            rpart[(wave * 8 + r) * 64 + lane] = racc_x[r];
+            rpart[(wave * 8 + 4 + r) * 64 + lane] = racc_y[r];
         }
     }
 
     __syncthreads();
-    if (drpb && tid < W) atomicAdd(drpb + head * W + tid, drpb_lds[tid]);
+    if (drpb) {
+        // thread (j, p): slot j, wave p/2, registers r = 2*(p&1), 2*(p&1)+1; the lane (n, g) whose register r
+        // holds slot j has n = 4g + r - shift + L - j (+32: merged block 2, +16: block 1)
+        const int j = tid & 31, p = tid >> 5, w = p >> 1;
+        float sum = 0.f;
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+            const int r = 2 * (p & 1) + rr;
+#pragma unroll
+            for (int gg = 0; gg < 4; ++gg) {
+                const int na = 4 * gg + r - shift + L - j;
+                const int nx = (NBV == 3 && na < 0) ? na + 32 : na, ny = na + 16;
+                if (nx >= 0 && nx < 16) sum += rpart[(w * 8 + r) * 64 + 16 * gg + nx];
+                if (ny >= 0 && ny < 16) sum += rpart[(w * 8 + 4 + r) * 64 + 16 * gg + ny];
+            }
+        }
+        rsum[p * 32 + j] = sum;
+    }
 
     // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
     // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb
@@ -712,8 +770,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             read_rows<C>(gop, gtile, qry_lane);
             const f32x4 s = dot_rows_mma<DT, C>(qop, kop);       // rows = queries 4g+r, col = key n
             const f32x4 dp = dot_rows_mma<DT, C>(gop, vop);
-            const f32x4 lse4 = *reinterpret_cast<LDS_PTR(f32x4)>((LDS_PTR(float))lse_lds + tq * 16 + 4 * g);
-            const f32x4 del4 = *reinterpret_cast<LDS_PTR(f32x4)>((LDS_PTR(float))delta_lds + tq * 16 + 4 * g);
+            const f32x4 lse4 = *reinterpret_cast<LDS_PTR(f32x4)>(lse_lds + tq * 16 + 4 * g);
+            const f32x4 del4 = *reinterpret_cast<LDS_PTR(f32x4)>(delta_lds + tq * 16 + 4 * g);
             float z[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) z[r] = __builtin_fmaf(s[r], scale2, bias2[vb][r]) - lse4[r];
@@ -750,28 +808,66 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             __builtin_amdgcn_raw_buffer_store_b64(wv, dvs, row_off + ct * 32 + g * 8, 0, 0);
         }
     }
+
+    if (drpb) {
+        __syncthreads();
+        if (tid < W) {
+            float t = 0.f;
+#pragma unroll
+            for (int p = 0; p < 8; ++p) t += rsum[p * 32 + tid];
+            if (drpb_partial)
+                drpb_partial[(size_t)item * kPartialStride + tid] = t;   // folded by drpb_reduce_kernel
+            else
+                atomicAdd(drpb + head * W + tid, t);
+        }
+    }
 }
 
 template <class DT, int C>
 int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
                const void *dout, const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g,
-               float scale, hipStream_t s) {
+               float scale, float *workspace, int64_t workspace_bytes, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, StripBwd<C>::kMaxTiles);
     if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    float *partial = nullptr;
+    if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
     auto kern = window_blocks(g) == 2 ? fused_bwd_kernel<DT, C, 2> : fused_bwd_kernel<DT, C, 3>;
-    kern<<<(unsigned)sp.items, kThreads, 0, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
+    const size_t lds = (size_t)(4 * sp.nt + 12) * Lds<C>::kTileBytes +
+                       (2 * (StripBwd<C>::kMaxTiles + 2) * 16 + 32 + (drpb ? kWaves * 8 * 64 + 8 * 32 : 0)) * sizeof(float);
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                                                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
                                                  t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
-                                                 sp.nt, sp.strips, scale);
+                                                 sp.nt, sp.strips, scale, partial);
+    if (partial)
+        drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();
+}
+
+template <class DT, int C>
+int64_t bwd_workspace(const Geom &g) {
+    return make_split(g.B, g.T, StripBwd<C>::kMaxTiles).items * kPartialStride * (int64_t)sizeof(float);
 }
 
 int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
               const void *out, const void *dout, const float *lse, const float *rpb, const int32_t *t_valid,
-              const Geom &g, float scale, int dtype, hipStream_t s) {
+              const Geom &g, float scale, int dtype, float *workspace, int64_t workspace_bytes, hipStream_t s) {
     (void)out;   // delta is recomputed from P and dP; O is not needed
     if (!window_blocks(g)) return NA1D_ERR_UNSUPPORTED;
-    NA1D_MFMA_DISPATCH(launch_bwd, dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, scale, s);
+    NA1D_MFMA_DISPATCH(launch_bwd, dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, scale, workspace,
+                       workspace_bytes, s);
+}
+
+int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype) {
+    if (!window_blocks(g)) return 0;
+    switch (g.C) {   // the split does not depend on the dtype
+        case 16: return bwd_workspace<BF16, 16>(g);
+        case 32: return bwd_workspace<BF16, 32>(g);
+        case 64: return bwd_workspace<BF16, 64>(g);
+        case 128: return bwd_workspace<BF16, 128>(g);
+    }
+    (void)dtype;
+    return 0;
 }
 
 int qk(float *, const void *, const void *, const Geom &, int, hipStream_t) { return NA1D_ERR_UNSUPPORTED; }

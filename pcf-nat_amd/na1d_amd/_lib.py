@@ -20,7 +20,8 @@ _i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_
 
 _UNFUSED = ("na1d_qk_forward", "na1d_av_forward", "na1d_q_backward", "na1d_k_backward",
             "na1d_a_backward", "na1d_v_backward")
-SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_version", "na1d_status_string")
+SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_backward_workspace_bytes",
+                      "na1d_version", "na1d_status_string")
 
 _lib = None
 
@@ -50,7 +51,9 @@ def load():
     lib.na1d_fused_forward.argtypes = [_ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                        _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _ptr]
     lib.na1d_fused_backward.restype = _int
-    lib.na1d_fused_backward.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _ptr]
+    lib.na1d_fused_backward.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _ptr, _i64, _ptr]
+    lib.na1d_fused_backward_workspace_bytes.restype = _i64
+    lib.na1d_fused_backward_workspace_bytes.argtypes = [_i64] * 6 + [_int]
     lib.na1d_version.restype = _int
     lib.na1d_version.argtypes = []
     lib.na1d_status_string.restype = ctypes.c_char_p
@@ -98,10 +101,20 @@ def call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, H, T, C, W, left, sca
     check(st, "na1d_fused_forward")
 
 
-def call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, B, H, T, C, W, left, scale):
+def fused_backward_workspace_bytes(B, H, T, C, W, left, dtype) -> int:
+    n = load().na1d_fused_backward_workspace_bytes(B, H, T, C, W, left, dtype_tag(dtype))
+    if n < 0:
+        check(int(n), "na1d_fused_backward_workspace_bytes")
+    return int(n)
+
+
+def call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, B, H, T, C, W, left, scale,
+                        workspace=None):
+    """``workspace``: optional uint8/any CUDA tensor used for the d rpb reduction."""
     lib = load()
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with torch.cuda.device(dq.device):
         st = lib.na1d_fused_backward(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(out), _p(dout),
                                      _p(lse), _p(rpb), _p(t_valid), B, H, T, C, W, left, scale,
-                                     dtype_tag(q.dtype), _stream(dq))
+                                     dtype_tag(q.dtype), _p(workspace), ws_bytes, _stream(dq))
     check(st, "na1d_fused_backward")

@@ -76,8 +76,14 @@ def test_fused_entry_points_validate():
     assert f(ok, None, ok, ok, ok, None, None, 4, 2, 8, 20, 5, 2, 1.0, 0, None) == -3
     assert f(None, None, None, None, None, None, None, 0, 1, 8, 16, 5, 2, 1.0, 0, None) == 0
     b = lib.na1d_fused_backward
-    assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, None, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, None) == -1  # lse
-    assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 90, 2, 1.0, 0, None) == -4
+    assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, None, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, None, 0, None) == -1  # lse
+    assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 90, 2, 1.0, 0, None, 0, None) == -4
+    assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, P(0x1008), 64, None) == -6
+    w = lib.na1d_fused_backward_workspace_bytes
+    assert w(4096, 16, 100, 16, 27, 13, 0) == 4096 * 32 * 4      # one 32-float row per work item
+    assert w(1024, 8, 300, 32, 15, 7, 1) > 0
+    assert w(4, 2, 8, 24, 5, 2, 0) == 0                          # generic kernel: no workspace
+    assert w(4, 3, 8, 16, 5, 2, 0) == -5 and w(4, 2, 8, 16, 99, 2, 0) == -4
 
 
 def test_python_layer_mirrors_reference_entry_points():

@@ -248,6 +248,23 @@ def test_model_shape_properties_at_full_size(dtype):
     assert (ones.float() - 1).abs().max().item() < (2e-2 if dtype == torch.bfloat16 else 4e-3)
 
 
+def test_deterministic_rpb_gradient_is_bit_reproducible():
+    """With deterministic=True d rpb is folded in a fixed order: two runs give the same bits, and the
+    atomics path agrees with it to fp32 rounding."""
+    N, H, T, C, W, L = 16, 16, 100, 16, 27, 13
+    q, k, v, do = make_inputs(N * H, T, C, W, 71, torch.float16, n=4, scale=0.25)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(5)) * 0.3
+    grads = []
+    for det in (True, True, False):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        rd = rpb.cuda().requires_grad_(True)
+        na1d_fused(qd, kd, vd, W, L, rpb=rd, num_heads=H, deterministic=det).backward(do.cuda())
+        grads.append((rd.grad.clone(), qd.grad.clone(), kd.grad.clone(), vd.grad.clone()))
+    assert all(torch.equal(a, b) for a, b in zip(grads[0], grads[1]))
+    assert all(torch.equal(a, b) for a, b in zip(grads[0][1:], grads[2][1:]))       # dq, dk, dv: no atomics at all
+    assert torch.allclose(grads[0][0], grads[2][0], rtol=1e-4, atol=1e-4)
+
+
 def test_runs_on_the_current_stream():
     """Launches go to torch's current stream (the reference uses the legacy default
     stream; its data prefetcher runs a side stream, public/Utils.py:89-100)."""
