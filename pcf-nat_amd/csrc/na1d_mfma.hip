@@ -34,6 +34,8 @@
 // all loads in flight at once - buffer loads, so rows outside the sequence read
 // as zero, which is the band's zero fill - then, after one barrier, each wave
 // computes tiles wave, wave+4, ... entirely out of LDS.
+#include <algorithm>
+
 #include "na1d_common.h"
 
 namespace na1d {
@@ -509,14 +511,14 @@ int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v
 // the row sum of the same registers, so O is never read.  Two passes over the
 // strip, both entirely out of LDS:
 //   pass 1, per query tile (plus one halo tile each side): S^T, dP^T in the
-//     "query = lane%16" layout -> P, delta, dS -> dQ^T = K^T . dS^T; delta goes to LDS.
-//   pass 2, per key block: S, dP with the operands swapped ("key = lane%16",
-//     queries 4g+r), P and dS recomputed with lse/delta of those queries, and
-//     dV^T += dO^T . P, dK^T += Q^T . dS accumulate in registers over the NBV query
-//     tiles that see the block - a gather over the inverse neighbourhood, no
-//     atomics, each output row written once.
-// The score work is done twice so that both contractions find their B operand
-// already in accumulator layout and nothing is exchanged between waves.
+//     "query = lane%16" layout -> P, delta, dS -> dQ^T = K^T . dS^T.  The rounded
+//     P and dS tiles stay in registers until every wave is done with K and V.
+//   Then they are written over the K/V regions as 16x16 tiles [query][key slot],
+//   and pass 2, per key block, reads them back transposed (ds_read_b64_tr_b16) as
+//     the B operands of dV^T += dO^T . P and dK^T += Q^T . dS, accumulating in
+//     registers over the NBV query tiles that see the block - a gather over the
+//     inverse neighbourhood, no atomics, each output row written once, and no
+//     second evaluation of the scores.
 // d rpb partial sums: one row of kPartialStride floats per work item, folded in a
 // fixed order by a second kernel (one workgroup per head).
 constexpr int kPartialStride = 32;
@@ -550,24 +552,27 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
-                 int strips, float scale, float *__restrict__ drpb_partial) {
+                 int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
     constexpr int kRowsQ = (MT + 2) * 16;
+    constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
+    constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
     static_assert(kRowsQ <= kThreads, "one thread per staged lse row");
-    // dynamic LDS (bwd_lds_bytes): K, V regions of nt+4 tiles (rows 16*i0 - 32 ...), Q, dO regions of nt+2 tiles
-    // (rows 16*i0 - 16 ...), lse and delta of the query-side rows, 32 bias floats, and - only when d rpb is
-    // wanted - per-lane partial sums and 8 partial sums per slot
+    // dynamic LDS (see launch_bwd): [K region | V region] of nt+4 tiles each (rows 16*i0 - 32 ...), reused after
+    // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt+2 tiles (rows 16*i0 - 16 ...); lse
+    // of the query-side rows; 32 bias floats; and - only when d rpb is wanted - per-lane partial sums and 8
+    // partial sums per slot
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = (nt + 4) * LL::kTileBytes, qry_region = (nt + 2) * LL::kTileBytes;
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
-    LDS_PTR(char) q_lds = v_lds + key_region;
+    LDS_PTR(char) sc_lds = k_lds;                  // score tiles [(tq*2 + X/Y)*2 + P/dS]
+    LDS_PTR(char) q_lds = k_lds + kv_bytes;
     LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
     LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
-    LDS_PTR(float) delta_lds = lse_lds + kRowsQ;
-    LDS_PTR(float) bias_lds = delta_lds + kRowsQ;
+    LDS_PTR(float) bias_lds = lse_lds + kRowsQ;
     LDS_PTR(float) rpart = bias_lds + 32;          // [kWaves * 8][64]
     LDS_PTR(float) rsum = rpart + kWaves * 8 * 64; // [8][32]
 
@@ -620,15 +625,16 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     Window<NBV> win;
     make_window<NBV>(win, bias_lds, W, L, shift, g, n);
 
-    // ---------------- pass 1: query tiles i0-1 .. i1 -> delta, dQ, drpb ----------------
+    // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
     const Rsrc dqs = make_rsrc(dq + seq_off, seq_bytes);
-    for (int qt = i0 - 1 + wave; qt <= i1; qt += kWaves) {
-        const int tq = qt - (i0 - 1);                       // tile index inside the query-side regions
-        if (qt < 0 || qt >= tiles) {                        // nothing there: its delta must still read as 0
-            if (g == 0) delta_lds[tq * 16 + n] = 0.f;
-            continue;
-        }
+    u32x2 sc[TPW][2][2];                // [tile of this wave][X/Y slot set][P / dS], rounded to 16 bit
+#pragma unroll
+    for (int jt = 0; jt < TPW; ++jt) {
+        sc[jt][0][0] = sc[jt][0][1] = sc[jt][1][0] = sc[jt][1][1] = u32x2{0u, 0u};
+        const int tq = wave + jt * kWaves;                  // tile index inside the query-side regions
+        const int qt = i0 - 1 + tq;
+        if (qt > i1 || qt < 0 || qt >= tiles) continue;     // nothing there: its scores stay zero
         RowOperand<C> qop, gop;
         read_rows<C>(qop, q_lds + tq * LL::kTileBytes, qry_lane);
         read_rows<C>(gop, g_lds + tq * LL::kTileBytes, qry_lane);
@@ -672,20 +678,26 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             part = __builtin_fmaf(py[r], dpy[r], part);
         }
         const float delta = xor_sum(part);
-        if (g == 0) delta_lds[tq * 16 + n] = delta;
-        if (qt < i0 || qt >= i1) continue;                  // halo tile: only its delta is needed
-
         float dsx[4], dsy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             dsx[r] = px[r] * (dpx[r] - delta);
             dsy[r] = py[r] * (dpy[r] - delta);
+        }
+        sc[jt][0][0] = u32x2{Mma<DT>::pack(px[0], px[1]), Mma<DT>::pack(px[2], px[3])};
+        sc[jt][1][0] = u32x2{Mma<DT>::pack(py[0], py[1]), Mma<DT>::pack(py[2], py[3])};
+        sc[jt][0][1] = u32x2{Mma<DT>::pack(dsx[0], dsx[1]), Mma<DT>::pack(dsx[2], dsx[3])};
+        sc[jt][1][1] = u32x2{Mma<DT>::pack(dsy[0], dsy[1]), Mma<DT>::pack(dsy[2], dsy[3])};
+        if (qt < i0 || qt >= i1) continue;                  // halo tile: only its scores are needed
+
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
             racc_x[r] += dsx[r];
             racc_y[r] += dsy[r];
         }
-        const u32x2 pkx = {Mma<DT>::pack(dsx[0], dsx[1]), Mma<DT>::pack(dsx[2], dsx[3])};
+        const u32x2 pkx = sc[jt][0][1];
         u32x2 db[NBV];
-        db[1] = u32x2{Mma<DT>::pack(dsy[0], dsy[1]), Mma<DT>::pack(dsy[2], dsy[3])};
+        db[1] = sc[jt][1][1];
         if (NBV == 3) {
             db[0] = u32x2{pkx.x & win.keep0.x, pkx.y & win.keep0.y};
             db[NBV - 1] = u32x2{pkx.x & win.keep2.x, pkx.y & win.keep2.y};
@@ -720,7 +732,17 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
 
-    __syncthreads();
+    __syncthreads();                    // every wave is done with K and V: their regions become the score tiles
+#pragma unroll
+    for (int jt = 0; jt < TPW; ++jt) {
+        const int tq = wave + jt * kWaves;
+        if (tq > nt + 1) continue;
+        LDS_PTR(char) t = sc_lds + tq * 4 * kScoreTile + n * 32 + g * 8;     // tile[query n][key slots 4g..4g+3]
+#pragma unroll
+        for (int xy = 0; xy < 2; ++xy)
+#pragma unroll
+            for (int pd = 0; pd < 2; ++pd) *reinterpret_cast<LDS_PTR(u32x2)>(t + (xy * 2 + pd) * kScoreTile) = sc[jt][xy][pd];
+    }
     if (drpb) {
         // thread (j, p): slot j, wave p/2, registers r = 2*(p&1), 2*(p&1)+1; the lane (n, g) whose register r
         // holds slot j has n = 4g + r - shift + L - j (+32: merged block 2, +16: block 1)
@@ -739,57 +761,43 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
         rsum[p * 32 + j] = sum;
     }
+    __syncthreads();
 
     // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
-    // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb
-    float bias2[NBV][4];
+    // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb.  Lane (n, g)
+    // of the transposed score read holds tile[query 4g+r][key slot n]; in a merged tile that entry belongs to
+    // block 0 when n - (4g+r) - shift + L >= 0 and to block 2 otherwise.
+    u32x2 keep0t = {0xffffffffu, 0xffffffffu};
+    if (NBV == 3) {
+        uint32_t m[4];
 #pragma unroll
-    for (int vb = 0; vb < NBV; ++vb)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) bias2[vb][r] = bias_at(bias_lds, 16 * vb - shift + n - (4 * g + r) + L, W);
+        for (int r = 0; r < 4; ++r) m[r] = (n - (4 * g + r) - shift + L >= 0) ? 0xffffu : 0u;
+        keep0t = u32x2{m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
+    }
+    const int sc_lane = (4 * g + (n >> 2)) * 32 + (n & 3) * 8;       // transposed read of a score tile
     const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
     const Rsrc dks = make_rsrc(dk + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
     const Rsrc dvs = make_rsrc(dv + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
     const int kp_lo = i0 + (shift == 16 ? 1 : 0), kp_hi = i1 - (shift == 0 ? 1 : 0);
     for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
-        RowOperand<C> kop, vop;
-        read_rows<C>(kop, k_lds + (kp - i0) * LL::kTileBytes, key_lane);
-        read_rows<C>(vop, v_lds + (kp - i0) * LL::kTileBytes, key_lane);
         f32x4 acck[CT], accv[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acck[ct] = accv[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const int key = 16 * kp - shift + n;
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
-            const int qt = kp - vb;
-            const int tq = qt - (i0 - 1);
+            const int tq = kp - vb - (i0 - 1);
             LDS_PTR(char) qtile = q_lds + tq * LL::kTileBytes;
             LDS_PTR(char) gtile = g_lds + tq * LL::kTileBytes;
-            RowOperand<C> qop, gop;
-            read_rows<C>(qop, qtile, qry_lane);
-            read_rows<C>(gop, gtile, qry_lane);
-            const f32x4 s = dot_rows_mma<DT, C>(qop, kop);       // rows = queries 4g+r, col = key n
-            const f32x4 dp = dot_rows_mma<DT, C>(gop, vop);
-            const f32x4 lse4 = *reinterpret_cast<LDS_PTR(f32x4)>(lse_lds + tq * 16 + 4 * g);
-            const f32x4 del4 = *reinterpret_cast<LDS_PTR(f32x4)>(delta_lds + tq * 16 + 4 * g);
-            float z[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) z[r] = __builtin_fmaf(s[r], scale2, bias2[vb][r]) - lse4[r];
-            if (16 * kp - shift < 0 || 16 * kp - shift + 16 > tv || 16 * qt + 16 > tv) {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int qrow = 16 * qt + 4 * g + r;
-                    z[r] += ((uint32_t)key >= (uint32_t)tv || qrow >= tv) ? mask2 : 0.f;
-                }
+            LDS_PTR(char) stile = sc_lds + (tq * 4 + (vb == 1 ? 2 : 0)) * kScoreTile + sc_lane;
+            u32x2 pb = read_tr(stile), db = read_tr(stile + kScoreTile);
+            if (NBV == 3 && vb == 0) {
+                pb = u32x2{pb.x & keep0t.x, pb.y & keep0t.y};
+                db = u32x2{db.x & keep0t.x, db.y & keep0t.y};
             }
-            float pp[4], ds[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                pp[r] = __builtin_amdgcn_exp2f(z[r]);
-                ds[r] = pp[r] * (dp[r] - del4[r]);
+            if (NBV == 3 && vb == 2) {
+                pb = u32x2{pb.x & ~keep0t.x, pb.y & ~keep0t.y};
+                db = u32x2{db.x & ~keep0t.x, db.y & ~keep0t.y};
             }
-            const u32x2 pb = {Mma<DT>::pack(pp[0], pp[1]), Mma<DT>::pack(pp[2], pp[3])};
-            const u32x2 db = {Mma<DT>::pack(ds[0], ds[1]), Mma<DT>::pack(ds[2], ds[3])};
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 accv[ct] = Mma<DT>::k16(read_tr(gtile + qry_tr.off[ct]), pb, accv[ct]);
@@ -809,17 +817,14 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
 
-    if (drpb) {
-        __syncthreads();
-        if (tid < W) {
-            float t = 0.f;
+    if (drpb && tid < W) {              // rsum was complete at the barrier before pass 2
+        float t = 0.f;
 #pragma unroll
-            for (int p = 0; p < 8; ++p) t += rsum[p * 32 + tid];
-            if (drpb_partial)
-                drpb_partial[(size_t)item * kPartialStride + tid] = t;   // folded by drpb_reduce_kernel
-            else
-                atomicAdd(drpb + head * W + tid, t);
-        }
+        for (int p = 0; p < 8; ++p) t += rsum[p * 32 + tid];
+        if (drpb_partial)
+            drpb_partial[(size_t)item * kPartialStride + tid] = t;   // folded by drpb_reduce_kernel
+        else
+            atomicAdd(drpb + head * W + tid, t);
     }
 }
 
@@ -832,13 +837,15 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     float *partial = nullptr;
     if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
     auto kern = window_blocks(g) == 2 ? fused_bwd_kernel<DT, C, 2> : fused_bwd_kernel<DT, C, 3>;
-    const size_t lds = (size_t)(4 * sp.nt + 12) * Lds<C>::kTileBytes +
-                       (2 * (StripBwd<C>::kMaxTiles + 2) * 16 + 32 + (drpb ? kWaves * 8 * 64 + 8 * 32 : 0)) * sizeof(float);
+    // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
+    const int kv_bytes = std::max(2 * (sp.nt + 4) * Lds<C>::kTileBytes, (sp.nt + 2) * 4 * 512);
+    const size_t lds = (size_t)kv_bytes + (size_t)2 * (sp.nt + 2) * Lds<C>::kTileBytes +
+                       ((StripBwd<C>::kMaxTiles + 2) * 16 + 32 + (drpb ? kWaves * 8 * 64 + 8 * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                                                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
                                                  t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
-                                                 sp.nt, sp.strips, scale, partial);
+                                                 sp.nt, sp.strips, scale, partial, kv_bytes);
     if (partial)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();
