@@ -20,8 +20,9 @@ class _FusedNA1D(torch.autograd.Function):
         assert q.dim() == 3 and q.shape == k.shape == v.shape, "q, k, v must all be [B, T, C]"
         B, T, C = q.shape
         assert B % num_heads == 0
+        ctx.rpb_shape = None if rpb is None else rpb.shape
         if rpb is not None:
-            rpb = rpb.reshape(num_heads, win_size).to(torch.float32).contiguous()
+            rpb = rpb.detach().reshape(num_heads, win_size).to(torch.float32).contiguous()
         if t_valid is not None:
             assert t_valid.numel() == B // num_heads
             t_valid = t_valid.to(device=q.device, dtype=torch.int32).contiguous()
@@ -48,6 +49,8 @@ class _FusedNA1D(torch.autograd.Function):
                     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
         _lib.call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid,
                                  B, num_heads, T, C, win_size, left, scale, workspace=ws)
+        if drpb is not None:
+            drpb = drpb.view(ctx.rpb_shape)
         return dq, dk, dv, drpb, None, None, None, None, None, None
 
 

@@ -1,0 +1,437 @@
+"""The callers of the NA1D operator: PCF-NAT and MFA-NAT speaker-embedding models.
+
+A compact restatement of the reference's model definitions
+(models/PCF_NATransformer.py, models/MFA_NATransformer.py, models/Modules.py,
+models/Pooling.py, models/SoftMaxLoss.py:99-138) in plain torch.nn, built so that
+
+* module and parameter names match the reference's ``state_dict`` (a reference
+  checkpoint loads with ``load_state_dict``);
+* the neighbourhood attention runs through this package's operator:
+  ``na="fused"`` (one HIP kernel each way, no mask or score tensor),
+  ``na="unfused"`` (the reference's own chain QK -> +rpb -> +mask -> softmax -> AV
+  through the drop-in Functions), or any callable with the signature of
+  :func:`na1d_amd.na1d_fused` (tests pass a CPU function here to build a twin).
+
+One class covers both families: PCF-NAT keeps activations channels-first
+``[N, C, T]`` with grouped 1x1 convolutions and one patch embedding per block
+whose output is added to the previous block's (PCF_NATransformer.py:443-448);
+MFA-NAT keeps them tokens-first ``[N, T, C]`` with linear layers
+(MFA_NATransformer.py:446-456).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .fused import na1d_fused
+from .nattn import getNA1dFunction
+
+MASK_VALUE = -100.0   # PCF_NATransformer.py:98
+
+
+# --------------------------------------------------------------------------- small pieces
+def sinusoid_table(dim, max_len, channels_first):
+    """Modules.py:38-56: even channels sin(pos * 10000^(c/dim)), odd channels cos (note: *, not /)."""
+    pos = torch.arange(max_len, dtype=torch.float32)
+    c = torch.arange(dim, dtype=torch.float32)
+    rate = torch.pow(torch.tensor(10000.0), c / dim)
+    table = pos.unsqueeze(1) * rate.unsqueeze(0)                          # [max_len, dim]
+    table = torch.where((torch.arange(dim) % 2 == 0).unsqueeze(0), torch.sin(table), torch.cos(table))
+    return table.t().unsqueeze(0) if channels_first else table.unsqueeze(0)
+
+
+class TokenBatchNorm(nn.Module):
+    """BatchNorm1d over the last dim of [N, T, C] (Modules.py:26-35)."""
+
+    def __init__(self, dim):
+        super().__init__()
+        self.norm = nn.BatchNorm1d(dim)
+
+    def forward(self, x):
+        return self.norm(x.transpose(-2, -1)).transpose(-2, -1) if x.dim() >= 3 else self.norm(x)
+
+
+class DropPath(nn.Module):
+    def __init__(self, p):
+        super().__init__()
+        self.drop_prob = p
+
+    def forward(self, x):
+        if self.drop_prob == 0.0 or not self.training:
+            return x
+        keep = 1 - self.drop_prob
+        mask = (keep + torch.rand((x.shape[0],) + (1,) * (x.dim() - 1), dtype=x.dtype, device=x.device)).floor_()
+        return x.div(keep) * mask
+
+
+class TDNNBlock(nn.Module):
+    """conv -> ReLU -> BatchNorm (Modules.py:15-23)."""
+
+    def __init__(self, cin, cout, kernel_size=1):
+        super().__init__()
+        self.conv = nn.Conv1d(cin, cout, kernel_size, padding="same")
+        self.activation = nn.ReLU(inplace=True)
+        self.norm = nn.BatchNorm1d(cout)
+
+    def forward(self, x):
+        return self.norm(self.activation(self.conv(x)))
+
+
+def _length_mask(shape, lens):
+    n, _, t = shape
+    count = torch.round(lens * t).view(n, 1, 1)
+    return torch.arange(t, device=lens.device).expand(n, 1, t) < count, count
+
+
+class AttentiveStatisticsPooling(nn.Module):
+    """Pooling.py:16-59 (global context on)."""
+
+    def __init__(self, channels, attention_channels=128):
+        super().__init__()
+        self.eps = 1e-12
+        self.tdnn = TDNNBlock(channels * 3, attention_channels, 1)
+        self.tanh = nn.Tanh()
+        self.conv = nn.Conv1d(attention_channels, channels, 1, padding="same")
+
+    def forward(self, x, lens=None):
+        if lens is None:
+            mask = None
+            mean = x.mean(-1, keepdim=True)
+            std = torch.sqrt(x.var(-1, keepdim=True).clamp(self.eps))
+        else:
+            mask, count = _length_mask(x.shape, lens)
+            mean = (x * mask).sum(-1, keepdim=True) / count
+            std = torch.sqrt((((x - mean).pow(2) * mask).sum(-1, keepdim=True) / count).clamp(self.eps))
+        ctx = torch.cat([x, mean.expand_as(x), std.expand_as(x)], dim=1)
+        w = self.conv(self.tanh(self.tdnn(ctx)))
+        if mask is not None:
+            w = w.masked_fill(mask == 0, -torch.inf)
+        w = F.softmax(w, dim=-1)
+        mean = (w * x).sum(-1, keepdim=True)
+        std = torch.sqrt((w * (x - mean).pow(2)).sum(-1, keepdim=True).clamp(self.eps))
+        return torch.cat((mean, std), dim=1).squeeze(-1)
+
+
+class StatisticsPooling(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.eps = 1e-12
+
+    def forward(self, x, lens=None):
+        if lens is None:
+            mean = x.mean(-1, keepdim=True)
+            std = torch.sqrt(x.var(-1, keepdim=True).clamp(self.eps))
+        else:
+            mask, count = _length_mask(x.shape, lens)
+            mean = (x * mask).sum(-1, keepdim=True) / count
+            std = torch.sqrt((((x - mean).pow(2) * mask).sum(-1, keepdim=True) / count).clamp(self.eps))
+        return torch.cat([mean, std], dim=1).squeeze(-1)
+
+
+# --------------------------------------------------------------------------- attention
+class _Projection(nn.Module):
+    """Per-token affine map on either layout: grouped 1x1 conv on [N,C,T] or Linear on [N,T,C]."""
+
+    @staticmethod
+    def make(cin, cout, bias, groups, channels_first):
+        return nn.Conv1d(cin, cout, 1, bias=bias, groups=groups) if channels_first else nn.Linear(cin, cout, bias=bias)
+
+
+def _split_heads(x, num_heads, groups, channels_first):
+    """qkv projection output -> contiguous [3, N*H, T, hd] (PCF :126-139, MFA :127-137)."""
+    if channels_first:
+        n, c3, t = x.shape
+        c = c3 // 3
+        x = x.view(n, c // groups, groups, 3, t).transpose(1, 2).contiguous().view(n, num_heads, c // num_heads, 3, t)
+        x = x.permute(3, 0, 1, 4, 2)
+    else:
+        n, t, c3 = x.shape
+        c = c3 // 3
+        x = x.view(n, t, 3, num_heads, c // num_heads).permute(2, 0, 3, 1, 4)
+    return x.contiguous().view(3, n * num_heads, t, c // num_heads)
+
+
+def _merge_heads(x, n, num_heads, channels_first):
+    """[N*H, T, hd] -> [N, C, T] or [N, T, C] (PCF :151-152, MFA :150-151)."""
+    _, t, hd = x.shape
+    x = x.view(n, num_heads, t, hd)
+    if channels_first:
+        return x.transpose(2, 3).contiguous().view(n, num_heads * hd, t)
+    return x.transpose(1, 2).contiguous().view(n, t, num_heads * hd)
+
+
+def _window_mask(T, W, left, padding, dtype, device):
+    """[N, T, W] additive mask of PCF_NATransformer.py:87-99."""
+    if padding is None:
+        padding = torch.zeros(1, dtype=torch.int64, device=device)
+    tv = (T - padding.to(device=device, dtype=torch.int64)).view(-1, 1, 1)
+    t = torch.arange(T, device=device).view(1, T, 1)
+    key = t - left + torch.arange(W, device=device).view(1, 1, W)
+    bad = (t >= tv) | (key < 0) | (key >= tv)
+    return torch.zeros(bad.shape, dtype=dtype, device=device).masked_fill(bad, MASK_VALUE)
+
+
+class NAttention(nn.Module):
+    """Neighbourhood attention layer (PCF_NATransformer.py:44-178 / MFA_NATransformer.py:43-177)."""
+
+    def __init__(self, frames, dim, num_heads, win_size, groups=1, channels_first=True, dtype=torch.bfloat16,
+                 na="fused"):
+        super().__init__()
+        if isinstance(win_size, int):
+            assert win_size > 0
+            left = win_size - 1 - win_size // 2
+        else:
+            win_size, left = win_size
+        assert win_size <= 80 and 0 <= left < win_size
+        head_dim = dim // num_heads
+        assert dim % num_heads == 0 and head_dim % 8 == 0
+        self.win_size, self.left, self.dim, self.num_heads, self.groups = win_size, left, dim, num_heads, groups
+        self.channels_first, self.na = channels_first, na
+        self.scale = head_dim ** -0.5
+        self.qkv = _Projection.make(dim, dim * 3, True, groups, channels_first)
+        self.relative_position_bias = nn.Parameter(torch.zeros(1, num_heads, 1, win_size))
+        nn.init.normal_(self.relative_position_bias, mean=0.0, std=0.02)
+        self.proj = _Projection.make(dim, dim, True, groups, channels_first)
+        self.register_buffer("attn_mask", _window_mask(frames, win_size, left, None, torch.float32, "cpu").unsqueeze(1))
+        if na == "unfused":
+            self.NA1d_QK_Function, self.NA1d_AV_Function = getNA1dFunction(C=head_dim, dilation=1, dtype=dtype)
+
+    def forward(self, x, padding=None):
+        n = x.shape[0]
+        t = x.shape[-1] if self.channels_first else x.shape[1]
+        h, w, left = self.num_heads, self.win_size, self.left
+        q, k, v = _split_heads(self.qkv(x), h, self.groups, self.channels_first)
+        q = q * self.scale                                   # in the activation dtype, as the reference does (:141)
+        t_valid = None if padding is None else (t - padding).to(torch.int32)
+        if callable(self.na):
+            out = self.na(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h)
+        elif self.na == "fused":
+            out = na1d_fused(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h)
+        else:                                                # the reference's un-fused chain (:141-150)
+            attn = self.NA1d_QK_Function.apply(q, k, w, left, 1).view(n, h, t, w)
+            attn = attn + self.relative_position_bias
+            attn = attn + _window_mask(t, w, left, padding, x.dtype, x.device).unsqueeze(1)
+            attn = torch.softmax(attn.view(n * h, t, w), dim=-1)
+            out = self.NA1d_AV_Function.apply(attn, v, w, left, 1)
+        return self.proj(_merge_heads(out, n, h, self.channels_first))
+
+
+class GlobalAttention(nn.Module):
+    """Dense attention with an additive sinusoid input (PCF :181-225 / MFA :180-221)."""
+
+    def __init__(self, dim, num_heads, groups=1, channels_first=True):
+        super().__init__()
+        self.num_heads, self.groups, self.channels_first = num_heads, groups, channels_first
+        self.scale = (dim // num_heads) ** -0.5
+        self.linear_pos = _Projection.make(dim, dim, False, groups, channels_first)
+        self.qkv = _Projection.make(dim, dim * 3, True, groups, channels_first)
+        self.proj = _Projection.make(dim, dim, True, groups, channels_first)
+
+    def forward(self, x, pos_emb, attn_mask=None):
+        n = x.shape[0]
+        x = x + self.linear_pos(pos_emb.to(x.dtype))
+        q, k, v = _split_heads(self.qkv(x), self.num_heads, self.groups, self.channels_first)
+        t, hd = q.shape[1], q.shape[2]
+        q, k, v = (z.view(n, self.num_heads, t, hd) for z in (q, k, v))
+        attn = (q * self.scale) @ k.transpose(-2, -1)
+        if attn_mask is not None:
+            attn = attn + attn_mask
+        out = torch.softmax(attn, dim=-1) @ v
+        return self.proj(_merge_heads(out.reshape(n * self.num_heads, t, hd), n, self.num_heads, self.channels_first))
+
+
+class Mlp(nn.Module):
+    def __init__(self, dim, hidden, groups, channels_first):
+        super().__init__()
+        self.fc1 = _Projection.make(dim, hidden, True, groups, channels_first)
+        self.act = nn.GELU()
+        self.fc2 = _Projection.make(hidden, dim, True, groups, channels_first)
+
+    def forward(self, x):
+        return self.fc2(self.act(self.fc1(x)))
+
+
+class NATFLayer(nn.Module):
+    """norm -> attention -> residual; norm -> MLP -> residual (PCF :228-265)."""
+
+    def __init__(self, frames, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na, mlp_ratio=4):
+        super().__init__()
+        self.local = isinstance(win_size, list) or win_size > 0
+        if self.local:
+            self.attn = NAttention(frames, dim, num_heads, win_size, groups, channels_first, dtype, na)
+        else:
+            self.attn = GlobalAttention(dim, num_heads, groups, channels_first)
+        norm = nn.BatchNorm1d if channels_first else TokenBatchNorm
+        self.norm1 = norm(dim)
+        self.drop_path = DropPath(drop_path) if drop_path > 0.0 else nn.Identity()
+        self.mlp = Mlp(dim, int(dim * mlp_ratio), groups, channels_first)
+        self.norm2 = norm(dim)
+
+    def forward(self, x, padding=None, pos_emb=None, attn_mask_global=None):
+        y = self.norm1(x)
+        y = self.attn(y, padding=padding) if self.local else self.attn(y, pos_emb=pos_emb, attn_mask=attn_mask_global)
+        x = x + self.drop_path(y)
+        return x + self.drop_path(self.mlp(self.norm2(x)))
+
+
+class NATFBlock(nn.Module):
+    def __init__(self, frames, depth, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na,
+                 use_checkpoint=False):
+        super().__init__()
+        pick = lambda v, i: v[i] if isinstance(v, list) else v
+        self.use_checkpoint = use_checkpoint if isinstance(use_checkpoint, list) else [use_checkpoint] * depth
+        self.blocks = nn.ModuleList([
+            NATFLayer(frames, dim, pick(num_heads, i), pick(win_size, i), pick(groups, i), pick(drop_path, i),
+                      channels_first, dtype, na) for i in range(depth)])
+
+    def forward(self, x, padding=None, pos_emb=None, attn_mask_global=None):
+        for layer, ckpt in zip(self.blocks, self.use_checkpoint):
+            if ckpt and self.training:      # activation checkpointing re-enters the operator's forward in backward
+                x = torch.utils.checkpoint.checkpoint(layer, x, padding, pos_emb, attn_mask_global, use_reentrant=False)
+            else:
+                x = layer(x, padding=padding, pos_emb=pos_emb, attn_mask_global=attn_mask_global)
+        return x
+
+
+class PatchEmbed(nn.Module):
+    def __init__(self, in_chans, embed_dim, patch_size, groups, channels_first):
+        super().__init__()
+        self.channels_first = channels_first
+        self.proj = nn.Conv1d(in_chans, embed_dim, kernel_size=patch_size, stride=patch_size, groups=groups)
+        self.norm = nn.BatchNorm1d(embed_dim)
+
+    def forward(self, x):
+        x = self.norm(self.proj(x))
+        return x if self.channels_first else x.transpose(1, 2)
+
+
+# --------------------------------------------------------------------------- the two model families
+class _NATransformer(nn.Module):
+    def __init__(self, channels_first, frames=300, patch_size=2, in_chans=80, output_emb_size=192, embed_dim=256,
+                 depths=(4, 4, 4, 4), num_heads=None, win_size=None, groups=(8, 4, 2, 1), drop_path_rate=0.0,
+                 proj_channel=1536, asp=True, poolnorm=True, use_checkpoint=False, dtype=torch.bfloat16, na="fused"):
+        super().__init__()
+        depths = list(depths)
+        nb = len(depths)
+        self.channels_first, self.frames, self.patch_size, self.embed_dim, self.num_blocks = \
+            channels_first, frames, patch_size, embed_dim, nb
+        emb_frames = frames // patch_size
+        pick = lambda v, i: v[i] if isinstance(v, (list, tuple)) else v
+        if channels_first:
+            self.patch_embeds = nn.ModuleList(
+                [PatchEmbed(in_chans, embed_dim, patch_size, pick(groups, i), True) for i in range(nb)])
+        else:
+            self.patch_embed = PatchEmbed(in_chans, embed_dim, patch_size, 1, False)
+        flat = [w for blk in win_size for w in (blk if isinstance(blk, list) else [blk])]
+        self.attn_global = any(isinstance(w, int) and w < 1 for w in flat)
+        if self.attn_global:
+            self.register_buffer("pos_emb", sinusoid_table(embed_dim, emb_frames, channels_first))
+            self.pos_emb_eval = None
+        dpr = torch.linspace(0, drop_path_rate, sum(depths)).tolist()
+        self.blocks = nn.ModuleList([
+            NATFBlock(emb_frames, depths[i], embed_dim, pick(num_heads, i), pick(win_size, i),
+                      pick(groups, i) if channels_first else 1, dpr[sum(depths[:i]):sum(depths[:i + 1])],
+                      channels_first, dtype, na, pick(use_checkpoint, i)) for i in range(nb)])
+        self.norm = nn.BatchNorm1d(embed_dim * nb)
+        self.proj = TDNNBlock(embed_dim * nb, proj_channel, 1)
+        self.pool = AttentiveStatisticsPooling(proj_channel) if asp else StatisticsPooling()
+        self.pool_norm = nn.BatchNorm1d(proj_channel * 2) if poolnorm else nn.Identity()
+        self.fc = nn.Linear(proj_channel * 2, output_emb_size)
+        for m in self.modules():                                   # PCF :392-400
+            if isinstance(m, nn.Linear):
+                nn.init.normal_(m.weight, mean=0.0, std=0.02)
+                if m.bias is not None:
+                    nn.init.constant_(m.bias, 0)
+
+    def forward(self, x, lens=None):
+        """x: [N, in_chans, frames]; lens: relative lengths in (0, 1] or None.  Returns [N, output_emb_size]."""
+        tin = x.shape[-1]
+        assert self.frames == tin or not self.training
+        padding = None
+        if lens is not None:
+            padding = ((tin - torch.round(lens * tin)) // self.patch_size).to(torch.int64)
+        t = (tin - self.patch_size) // self.patch_size + 1
+        pos_emb = mask_global = None
+        if self.attn_global:
+            if self.training:
+                pos_emb = self.pos_emb
+            else:
+                if self.pos_emb_eval is None or self.pos_emb_eval.device != x.device:
+                    self.pos_emb_eval = sinusoid_table(self.embed_dim, 40000, self.channels_first).to(x.device)
+                pos_emb = self.pos_emb_eval[:, :, :t] if self.channels_first else self.pos_emb_eval[:, :t, :]
+                if padding is not None:
+                    pad = torch.arange(t, device=x.device).unsqueeze(0) >= (t - padding.to(x.device)).unsqueeze(1)
+                    both = pad.unsqueeze(-1) | pad.unsqueeze(-2)
+                    mask_global = torch.zeros(both.shape, dtype=x.dtype, device=x.device).masked_fill(both, MASK_VALUE)
+                    mask_global = mask_global.unsqueeze(1)
+        if padding is not None:
+            padding = padding.to(x.device)
+        outs = []
+        if self.channels_first:
+            y = None
+            for embed, block in zip(self.patch_embeds, self.blocks):
+                e = embed(x)
+                y = block(e if y is None else e + y, padding=padding, pos_emb=pos_emb, attn_mask_global=mask_global)
+                outs.append(y)
+            x = torch.cat(outs, dim=1)
+        else:
+            y = self.patch_embed(x)
+            for block in self.blocks:
+                y = block(y, padding=padding, pos_emb=pos_emb, attn_mask_global=mask_global)
+                outs.append(y)
+            x = torch.cat(outs, dim=-1).transpose(1, 2)
+        x = self.proj(self.norm(x))
+        return self.fc(self.pool_norm(self.pool(x, lens=lens)))
+
+
+class PCF_NATransformer(_NATransformer):
+    """models/PCF_NATransformer.py:319-462; defaults of configs/pcf_nat4x4.yaml:45-63."""
+
+    def __init__(self, depths=(4, 4, 4, 4), num_heads=None, win_size=None, **kw):
+        n = len(depths)
+        num_heads = num_heads or [[16] * (depths[i] - 1) + [4 if i % 2 == 0 else 16] for i in range(n)]
+        win_size = win_size or [[27] * (depths[i] - 1) + [0 if i % 2 == 0 else 27] for i in range(n)]
+        super().__init__(True, depths=depths, num_heads=num_heads, win_size=win_size, **kw)
+
+
+class MFA_NATransformer(_NATransformer):
+    """models/MFA_NATransformer.py:325-466; defaults of configs/mfa_nat4x4.yaml:45-62."""
+
+    def __init__(self, depths=(4, 4, 4, 4), num_heads=None, win_size=None, **kw):
+        n = len(depths)
+        num_heads = num_heads or [[16] * (depths[i] - 1) + [4 if i % 2 == 1 else 16] for i in range(n)]
+        win_size = win_size or [[27] * (depths[i] - 1) + [0 if i % 2 == 1 else 27] for i in range(n)]
+        kw.pop("groups", None)
+        super().__init__(False, depths=depths, num_heads=num_heads, win_size=win_size, groups=1, **kw)
+
+
+def pcf_nat_6x4(**kw):
+    """configs/pcf_nat6x4.yaml:45-63 (activation checkpointing on the first four layers of block 0)."""
+    kw.setdefault("use_checkpoint", [[True] * 4 + [False] * 2, False, False, False])
+    return PCF_NATransformer(depths=(6, 6, 6, 6), **kw)
+
+
+class ArcMarginSubCenters(nn.Module):
+    """AAM-softmax with sub-centres (models/SoftMaxLoss.py:99-138)."""
+
+    def __init__(self, emb_size=192, n_classes=5994, m=0.2, s=32.0, subcenters=3):
+        super().__init__()
+        self.s, self.m = s, m
+        self.W = nn.Parameter(torch.empty(n_classes, subcenters, emb_size))
+        nn.init.xavier_uniform_(self.W)
+        self.cos_m, self.sin_m = math.cos(m), math.sin(m)
+        self.th, self.mm = math.cos(math.pi - m), math.sin(math.pi - m) * m
+
+    def forward(self, x, labels):
+        cosine = torch.einsum("ne,cse->ncs", F.normalize(x, dim=-1), F.normalize(self.W, dim=-1)).amax(-1)
+        with torch.no_grad():
+            acc1 = (cosine.argmax(1) == labels).sum()
+        sine = torch.sqrt(1.0 - cosine.pow(2))
+        shifted = cosine * self.cos_m - sine * self.sin_m
+        shifted = torch.where(cosine > self.th, shifted, cosine - self.mm)
+        one_hot = F.one_hot(labels.long(), cosine.shape[1]).to(cosine.dtype)
+        logits = (one_hot * shifted + (1.0 - one_hot) * cosine) * self.s
+        return F.cross_entropy(logits, labels.long()), acc1

@@ -1,0 +1,114 @@
+"""BASELINE configs 3-5 at reduced batch: the GPU models (HIP operator, 16-bit autocast) against a CPU fp32
+twin with the same state_dict whose attention is the oracle.  Bars: embedding cosine >= 0.999."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import na1d_oracle as O
+from na1d_amd import models
+
+pytestmark = pytest.mark.gpu
+
+
+def oracle_na(q, k, v, W, L, rpb=None, t_valid=None, num_heads=1):
+    T = q.shape[1]
+    pad = None if t_valid is None else (T - t_valid).to(torch.int64)
+    return O.na1d_forward(q, k, v, W, L, rpb.reshape(num_heads, W), pad, num_heads)[0]
+
+
+def _randomise_norm_stats(model, seed):
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for k, v in model.state_dict().items():
+            if k.endswith("running_mean"):
+                v.copy_(torch.randn(v.shape, generator=g) * 0.1)
+            if k.endswith("running_var"):
+                v.copy_(torch.rand(v.shape, generator=g) * 0.5 + 0.75)
+
+
+def _twin(factory, dtype, seed=0, **kw):
+    torch.manual_seed(seed)
+    cpu = factory(na=oracle_na, dtype=dtype, **kw)
+    _randomise_norm_stats(cpu, seed)
+    return cpu
+
+
+@pytest.mark.parametrize("na", ["fused", "unfused"])
+def test_pcf_nat_4x4_inference_bf16(na):
+    """cfg3: 80-dim fbank, 200 frames, bf16; pooled speaker embedding vs the CPU twin."""
+    cpu = _twin(models.PCF_NATransformer, torch.bfloat16).eval()
+    gpu = models.PCF_NATransformer(na=na, dtype=torch.bfloat16)
+    gpu.load_state_dict(cpu.state_dict())
+    gpu = gpu.cuda().eval()
+    x = torch.randn(8, 80, 200, generator=torch.Generator().manual_seed(1))
+    x = x - x.mean(-1, keepdim=True)                       # CMN over time, as the evaluation harness does
+    with torch.no_grad():
+        want = cpu(x)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = gpu(x.cuda())
+    cos = F.cosine_similarity(got.float().cpu(), want, dim=-1)
+    assert got.shape == (8, 192)
+    assert cos.min().item() >= 0.999, cos
+
+
+def test_pcf_nat_6x4_variable_length_bf16():
+    """cfg4: lengths uniform in 300..2000 frames, padded to the longest, masks from `lens`."""
+    cpu = _twin(models.pcf_nat_6x4, torch.bfloat16).eval()
+    gpu = models.pcf_nat_6x4(na="fused", dtype=torch.bfloat16)
+    gpu.load_state_dict(cpu.state_dict())
+    gpu = gpu.cuda().eval()
+    g = torch.Generator().manual_seed(2)
+    frames = torch.randint(300, 2001, (4,), generator=g)
+    tmax = int(frames.max())
+    x = torch.randn(4, 80, tmax, generator=g)
+    for i, f in enumerate(frames):
+        x[i, :, f:] = 0
+    lens = frames.float() / tmax
+    with torch.no_grad():
+        want = cpu(x, lens)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = gpu(x.cuda(), lens.cuda())
+    cos = F.cosine_similarity(got.float().cpu(), want, dim=-1)
+    assert cos.min().item() >= 0.999, cos
+
+
+def test_mfa_nat_4x4_training_step_fp16():
+    """cfg5: forward+backward through NA1D under fp16 autocast with a GradScaler, AAM sub-centre head over
+    5994 classes, one SGD-Nesterov step; loss and parameter gradients vs the CPU fp32 twin."""
+    cpu = _twin(models.MFA_NATransformer, torch.float16, frames=200).train()
+    gpu = models.MFA_NATransformer(na="fused", dtype=torch.float16, frames=200)
+    gpu.load_state_dict(cpu.state_dict())
+    gpu = gpu.cuda().train()
+    torch.manual_seed(3)
+    head_cpu = models.ArcMarginSubCenters(192, 5994, m=0.2, s=32.0, subcenters=3)
+    head_gpu = models.ArcMarginSubCenters(192, 5994, m=0.2, s=32.0, subcenters=3)
+    head_gpu.load_state_dict(head_cpu.state_dict())
+    head_gpu = head_gpu.cuda()
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(8, 80, 200, generator=g)
+    labels = torch.randint(0, 5994, (8,), generator=g)
+
+    loss_cpu, _ = head_cpu(cpu(x), labels)
+    loss_cpu.backward()
+
+    opt = torch.optim.SGD(list(gpu.parameters()) + list(head_gpu.parameters()), lr=0.01, momentum=0.9, nesterov=True)
+    scaler = torch.amp.GradScaler("cuda", init_scale=1024.0)
+    with torch.autocast("cuda", dtype=torch.float16):
+        emb = gpu(x.cuda())
+    loss_gpu, _ = head_gpu(emb.float(), labels.cuda())
+    scaler.scale(loss_gpu).backward()
+    scaler.unscale_(opt)
+    assert abs(loss_gpu.item() - loss_cpu.item()) < 0.05 * abs(loss_cpu.item())
+    checked = 0
+    for (name, pc), pg in zip(cpu.named_parameters(), gpu.parameters()):
+        if pc.grad is None or pc.grad.norm() < 1e-6:
+            continue
+        if any(s in name for s in ("relative_position_bias", "qkv.weight", "fc.weight", "patch_embed.proj.weight")):
+            cos = F.cosine_similarity(pg.grad.float().cpu().flatten(), pc.grad.flatten(), dim=0).item()
+            assert cos > 0.98, (name, cos)
+            checked += 1
+    assert checked >= 20
+    before = gpu.fc.weight.detach().clone()
+    scaler.step(opt)
+    scaler.update()
+    assert not torch.equal(before, gpu.fc.weight.detach())

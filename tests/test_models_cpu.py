@@ -1,0 +1,71 @@
+"""The restated PCF-NAT / MFA-NAT callers against vectors written by the reference's own model
+code (tests/golden/make_model_golden.py): same state_dict, same inputs -> same embeddings.
+The attention itself runs through the CPU oracle here (the product has no CPU path); what this
+pins is everything around the operator - head split/merge, grouped projections, block
+composition, sinusoid table, pooling with lengths, parameter names."""
+import os
+
+import pytest
+import torch
+
+from oracle import na1d_oracle as O
+from na1d_amd import models
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+COMMON = dict(frames=24, patch_size=2, in_chans=10, output_emb_size=16, embed_dim=32, depths=[2, 2],
+              drop_path_rate=0.1, proj_channel=24, asp=True, poolnorm=True, dtype=torch.float32)
+CASES = {
+    "pcf": (models.PCF_NATransformer, dict(num_heads=[[4, 2], [4, 4]], win_size=[[5, 0], [[6, 2], 5]], groups=[2, 1])),
+    "mfa": (models.MFA_NATransformer, dict(num_heads=[[4, 4], [4, 2]], win_size=[[5, [6, 2]], [5, 0]])),
+}
+
+
+def oracle_na(q, k, v, W, L, rpb=None, t_valid=None, num_heads=1):
+    T = q.shape[1]
+    pad = None if t_valid is None else (T - t_valid).to(torch.int64)
+    return O.na1d_forward(q, k, v, W, L, rpb.reshape(num_heads, W), pad, num_heads)[0]
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_model_reproduces_reference_vectors(name):
+    cls, extra = CASES[name]
+    blob = torch.load(os.path.join(GOLD, "model_%s.pt" % name), weights_only=True)
+    model = cls(**COMMON, **extra, na=oracle_na)
+    missing, unexpected = model.load_state_dict(blob["state_dict"], strict=True), None
+    model.eval()
+    with torch.no_grad():
+        out_lens = model(blob["x"], blob["lens"])
+        out_full = model(blob["x"])
+    assert torch.allclose(out_lens, blob["out_lens"], atol=2e-5, rtol=1e-4)
+    assert torch.allclose(out_full, blob["out_full"], atol=2e-5, rtol=1e-4)
+    assert not torch.allclose(blob["out_lens"], blob["out_full"], atol=1e-3)      # the lengths matter
+
+
+def test_state_dict_names_match_reference():
+    blob = torch.load(os.path.join(GOLD, "model_pcf.pt"), weights_only=True)
+    cls, extra = CASES["pcf"]
+    ours = cls(**COMMON, **extra, na=oracle_na).state_dict()
+    assert list(ours.keys()) == list(blob["state_dict"].keys())
+    assert all(ours[k].shape == v.shape for k, v in blob["state_dict"].items())
+    assert "blocks.0.blocks.0.attn.relative_position_bias" in ours and "blocks.0.blocks.0.attn.attn_mask" in ours
+
+
+def test_full_size_layer_counts():
+    """configs/pcf_nat4x4.yaml, pcf_nat6x4.yaml, mfa_nat4x4.yaml: 14 NA + 2 global layers (4x4), 22 + 2 (6x4)."""
+    def count(m):
+        layers = [l for b in m.blocks for l in b.blocks]
+        return sum(l.local for l in layers), sum(not l.local for l in layers)
+    assert count(models.PCF_NATransformer()) == (14, 2)
+    assert count(models.MFA_NATransformer()) == (14, 2)
+    assert count(models.pcf_nat_6x4()) == (22, 2)
+    att = models.PCF_NATransformer().blocks[0].blocks[0].attn
+    assert (att.win_size, att.left, att.num_heads, att.dim // att.num_heads) == (27, 13, 16, 16)
+
+
+def test_first_step_loss_matches_published_log():
+    """results/mfa_nat4x4/epoch=1/loss_log.txt:1 records a first-step loss of 17.77 with 17 982 classes:
+    with random embeddings the AAM sub-centre loss sits near ln(n) + s*(margin terms) ~ 17-19."""
+    torch.manual_seed(0)
+    head = models.ArcMarginSubCenters(192, 17982, m=0.2, s=32.0, subcenters=3)
+    loss, _ = head(torch.randn(256, 192), torch.randint(0, 17982, (256,)))
+    assert 16.0 < loss.item() < 20.0
