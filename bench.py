@@ -114,6 +114,55 @@ def cpu_baseline(w, budget_s=15.0):
                       % (n_sample, w["N"], B, T, len(times), sec)}
 
 
+def oracle_attention(q, k, v, W, L, rpb=None, t_valid=None, num_heads=1):
+    """CPU attention for the baseline twin of the model (the product has no CPU path)."""
+    import torch
+    from oracle import na1d_oracle as O
+    pad = None if t_valid is None else (q.shape[1] - t_valid).to(torch.int64)
+    return O.na1d_forward(q, k, v, W, L, rpb.reshape(num_heads, W), pad, num_heads)[0]
+
+
+def model_inference(batch=256, frames=200, steps=10, warmup=3, cpu=True):
+    """PCF-NAT 4x4 inference (BASELINE config 3): bf16 autocast, random-init weights, 80-dim fbank-shaped
+    N(0,1) input with the mean over time removed, fused NA1D in all 14 NA layers.  Returns embeddings/s on the
+    GPU and, as a baseline, of the same model in PyTorch CPU fp32 on a bounded batch."""
+    import torch
+    from na1d_amd import models
+    torch.manual_seed(0)
+    twin = models.PCF_NATransformer(na=oracle_attention, dtype=torch.bfloat16).eval()
+    gpu = models.PCF_NATransformer(na="fused", dtype=torch.bfloat16)
+    gpu.load_state_dict(twin.state_dict())
+    gpu = gpu.cuda().eval()
+    x = torch.randn(batch, 80, frames, generator=torch.Generator().manual_seed(1))
+    x = x - x.mean(-1, keepdim=True)
+    xd = x.cuda()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        for _ in range(warmup):
+            out = gpu(xd)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            out = gpu(xd)
+        torch.cuda.synchronize()
+        sec = (time.perf_counter() - t0) / steps
+    res = {"model": "PCF-NAT 4x4", "batch": batch, "frames": frames, "dtype": "bf16", "steps": steps,
+           "ms_per_batch": round(sec * 1e3, 3), "embeddings_per_s": round(batch / sec, 1)}
+    if cpu:
+        threads = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(threads)
+        nb = 16
+        with torch.no_grad():
+            ref = twin(x[:nb])
+            t0 = time.perf_counter()
+            ref = twin(x[:nb])
+            csec = time.perf_counter() - t0
+        cos = torch.nn.functional.cosine_similarity(out[:nb].float().cpu(), ref, dim=-1).min().item()
+        res["cpu_baseline"] = {"embeddings_per_s": round(nb / csec, 2), "cores": threads, "kind": "port",
+                               "sample": "batch %d of %d, one timed pass after one warm-up, PyTorch CPU fp32" % (nb, batch)}
+        res["min_cosine_vs_cpu_twin"] = round(cos, 5)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -121,6 +170,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-model", action="store_true", help="skip the PCF-NAT 4x4 embeddings/s leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the op shards over "
@@ -226,6 +276,10 @@ def main():
     }
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(w)
+    if not args.no_model:
+        del sets
+        torch.cuda.empty_cache()
+        line["pcf_nat_4x4_inference"] = model_inference(cpu=not args.no_cpu_baseline)
     print(json.dumps(line))
 
 
