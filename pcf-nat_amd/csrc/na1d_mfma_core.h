@@ -1,0 +1,341 @@
+// Shared machinery of the MFMA (matrix-core) NA1D kernels for gfx950.
+//
+// Tiles.  A sequence is cut into 16-row tiles at multiples of 16.  A query tile
+// (rows t0 .. t0+15) meets keys t0-L .. t0+15+R, 15+W rows, which are covered by
+// NBV "virtual" key blocks of 16 consecutive rows starting at row t0 - shift:
+//   NBV = 2 (W <= 17): shift = L, the 32 rows start exactly at the first key;
+//   NBV = 3 (L, R <= 16, W <= 32): shift = 16.
+// The band product is then NBV 16x16 MFMA tiles
+//
+//   S^T[key, query] = K_blk (A: 16 keys x C) . Q_tile^T (B: C x 16 queries)
+//
+// The accumulator of v_mfma_f32_16x16x16 puts element (row 4g+r, col n) in lane
+// 16g+n, register r (g = lane/16, n = lane%16).  For S^T that is "query n, keys
+// 4g..4g+3": per-query quantities (row max, row sum, LSE) are lane-local up to a
+// reduction over g, and the same registers, rounded to 16 bit, are exactly the B
+// operand (k = key) of
+//
+//   O^T[chan, query] = V_blk^T (A: 16 chans x 16 keys) . P^T (B: 16 keys x 16 queries)
+//
+// so probabilities never leave registers.  V^T (and every other operand whose
+// contraction index runs along memory rows) comes from LDS through
+// ds_read_b64_tr_b16, which hands lane n of a 16-lane group column n of a 4x16
+// tile of 16-bit values whose rows the group's lanes addressed four lanes apiece.
+//
+// Lane (n, g) holds, for query n, virtual keys 16*vb + 4g + r, i.e. window slot
+// j = 16*vb + 4g + r - shift - n + L.  With three blocks and W <= 32 a lane never
+// needs block 0 and block 2 in the same register r (block 0 is in the band only
+// for 4g+r-n >= 16-L, block 2 only for 4g+r-n <= R-16), so the two are merged
+// into one set of four slots: every lane carries 8 score slots either way.
+//
+// Work.  A workgroup of four waves owns a strip of up to kMaxTiles<C> consecutive
+// tiles of one sequence.  It first copies the strip's rows of every operand
+// (plus one 16-row halo block each side for the key-side operands) into LDS with
+// all loads in flight at once - buffer loads, so rows outside the sequence read
+// as zero, which is the band's zero fill - then, after one barrier, each wave
+// computes tiles wave, wave+4, ... entirely out of LDS.
+#pragma once
+
+#include <algorithm>
+
+#include "na1d_common.h"
+
+namespace na1d {
+namespace mfma {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short i16x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+#define LDS_PTR(T) __attribute__((address_space(3))) T *
+
+#ifndef NA1D_WAVES
+#define NA1D_WAVES 4
+#endif
+constexpr int kWaves = NA1D_WAVES;   // waves per workgroup
+constexpr int kThreads = 64 * kWaves;
+constexpr float kNegInf = -__builtin_inff();
+
+// ---- per-dtype MFMA wrappers; operands travel as raw 32-bit registers --------
+template <class DT> struct Mma;
+template <> struct Mma<FP16> {
+    __device__ static inline f32x4 k16(u32x2 a, u32x2 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, a), __builtin_bit_cast(f16x4, b), c, 0, 0, 0);
+    }
+    __device__ static inline f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+    __device__ static inline uint32_t pack(float lo, float hi) {
+        f32x2 x = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
+    }
+};
+template <> struct Mma<BF16> {
+    __device__ static inline f32x4 k16(u32x2 a, u32x2 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4, a), __builtin_bit_cast(i16x4, b), c, 0, 0, 0);
+    }
+    __device__ static inline f32x4 k32(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+    __device__ static inline uint32_t pack(float lo, float hi) {
+        f32x2 x = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+    }
+};
+
+// ---- buffer resources -----------------------------------------------------------
+// Raw buffer resource over one sequence of one tensor: loads outside [0, bytes)
+// return zero and stores outside are dropped - no branches, no clamping.
+using Rsrc = __amdgpu_buffer_rsrc_t;
+__device__ inline Rsrc make_rsrc(const void *base, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
+}
+
+// ---- LDS layout -------------------------------------------------------------------
+// Rows of C 16-bit channels, row-major and unpadded; the 16-byte units of a row
+// are XOR-swizzled with the row's 256-byte phase so that the 16 rows an operand
+// read touches land in distinct banks.  The swizzle term repeats every 16 rows.
+template <int C> struct Lds {
+    static constexpr int kUnits = C / 8;                 // 16-byte units per row
+    static constexpr int kRowBytes = 2 * C;
+    static constexpr int kTileBytes = 16 * kRowBytes;
+    static constexpr int kRowsPerPhase = kUnits >= 16 ? 1 : 16 / kUnits;   // rows per 256 bytes
+    __device__ static inline int swz(int row) { return (row / kRowsPerPhase) & (kUnits - 1); }
+    // byte address of (row, byte-in-row)
+    __device__ static inline int addr(int row, int byte) {
+        return row * kRowBytes + ((((byte >> 4) ^ swz(row)) << 4) | (byte & 15));
+    }
+};
+
+// Tiles per strip (compile-time ceiling that sizes LDS and the copy loops).
+template <int C> struct Strip {
+    static constexpr int kMaxTiles = C <= 16 ? 8 : C <= 32 ? 8 : C <= 64 ? 4 : 2;
+};
+
+// Copy up to NTILES tiles of rows, starting at row_lo of a sequence, into an LDS
+// region, all loads in flight before the first LDS store.  Split in two so several
+// regions' loads can be issued back to back.  NTILES fixes the (unrolled) number of
+// loads per thread; the caller's buffer resource ends where the wanted rows end, so
+// surplus loads fetch nothing.
+template <int C, int NTILES> struct Stage {
+    static constexpr int kTotal = NTILES * 16 * Lds<C>::kUnits;             // 16-byte units
+    static constexpr int kRounds = (kTotal + kThreads - 1) / kThreads;
+    u32x4 x[kRounds];
+    __device__ inline void issue(Rsrc src, int row_lo, int tid) {
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j)
+            x[j] = __builtin_amdgcn_raw_buffer_load_b128(src, (row_lo * Lds<C>::kUnits + j * kThreads + tid) * 16, 0, 0);
+    }
+    // `ntiles` <= NTILES: the region only has room for that many tiles
+    __device__ inline void commit(LDS_PTR(char) region, int ntiles, int tid) const {
+        const int total = ntiles * 16 * Lds<C>::kUnits;
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int u = j * kThreads + tid;
+            if (u < total)
+                *reinterpret_cast<LDS_PTR(u32x4)>(region + Lds<C>::addr(u / Lds<C>::kUnits, (u % Lds<C>::kUnits) * 16)) = x[j];
+        }
+    }
+};
+
+// ---- operands out of LDS ------------------------------------------------------
+// Row operand (A or B of a contraction over channels): lane (n, g) holds row n of a
+// 16-row tile; a 32-wide step s covers channels 32s + 8g .. +7, the 16-wide
+// remainder channels 32*k32 + 4g .. +3.  Offsets are per-lane constants.
+template <int C> struct RowOperand {
+    static constexpr int k32 = C / 32;
+    static constexpr int k16 = (C % 32) / 16;
+    u32x4 w32[k32 > 0 ? k32 : 1];
+    u32x2 w16[k16 > 0 ? k16 : 1];
+};
+template <int C> struct RowLane {        // this lane's byte offsets for a row operand whose tile starts `row0` rows into a region
+    int off32[RowOperand<C>::k32 > 0 ? RowOperand<C>::k32 : 1];
+    int off16;
+    __device__ inline void init(int row0, int lane) {
+        const int g = lane >> 4, n = lane & 15;
+#pragma unroll
+        for (int s = 0; s < RowOperand<C>::k32; ++s) off32[s] = Lds<C>::addr(row0 + n, 64 * s + 16 * g);
+        off16 = Lds<C>::addr(row0 + n, 64 * RowOperand<C>::k32 + 8 * g);
+    }
+};
+template <int C>
+__device__ inline void read_rows(RowOperand<C> &o, LDS_PTR(char) tile, const RowLane<C> &l) {
+#pragma unroll
+    for (int s = 0; s < RowOperand<C>::k32; ++s) o.w32[s] = *reinterpret_cast<LDS_PTR(u32x4)>(tile + l.off32[s]);
+    if (RowOperand<C>::k16) o.w16[0] = *reinterpret_cast<LDS_PTR(u32x2)>(tile + l.off16);
+}
+template <class DT, int C>
+__device__ inline f32x4 dot_rows_mma(const RowOperand<C> &a, const RowOperand<C> &b) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < RowOperand<C>::k32; ++s) acc = Mma<DT>::k32(a.w32[s], b.w32[s], acc);
+    if (RowOperand<C>::k16) acc = Mma<DT>::k16(a.w16[0], b.w16[0], acc);
+    return acc;
+}
+
+// Transposed operand: output lane (n, g) receives tile[row 4g+0..3][chan 16*ct + n];
+// the lane supplies the address of row 4g + (n>>2), byte 32*ct + 8*(n&3).
+template <int C> struct TrLane {
+    int off[C / 16];
+    __device__ inline void init(int row0, int lane) {
+        const int g = lane >> 4, n = lane & 15;
+#pragma unroll
+        for (int ct = 0; ct < C / 16; ++ct) off[ct] = Lds<C>::addr(row0 + 4 * g + (n >> 2), 32 * ct + 8 * (n & 3));
+    }
+};
+__device__ inline u32x2 read_tr(LDS_PTR(char) p) {
+    return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(reinterpret_cast<LDS_PTR(i16x4)>(p)));
+}
+
+// ---- reductions over g = lane/16 (lanes n, n+16, n+32, n+48), result in all four ----
+// v_permlane16_swap / v_permlane32_swap exchange 16- and 32-lane rows between two
+// registers, so swapping a value with itself lines up each lane's partner.
+__device__ inline void swap_rows16(float x, float &a, float &b) {
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    a = __uint_as_float(r.x);
+    b = __uint_as_float(r.y);
+}
+__device__ inline void swap_rows32(float x, float &a, float &b) {
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    a = __uint_as_float(r.x);
+    b = __uint_as_float(r.y);
+}
+// Plain v_max_f32 / v_max3_f32: scores are never NaN, so the quieting that fmaxf()
+// adds in front of every operand is skipped.
+__device__ inline float max2(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+__device__ inline float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ inline float xor_max(float x) {
+    float a, b;
+    swap_rows16(x, a, b);
+    swap_rows32(max2(a, b), a, b);
+    return max2(a, b);
+}
+__device__ inline float xor_sum(float x) {
+    float a, b;
+    swap_rows16(x, a, b);
+    swap_rows32(a + b, a, b);
+    return a + b;
+}
+
+// ---- window slots of a lane ------------------------------------------------------
+template <int NBV> struct Window {
+    // slot sets: X = block 0 (NBV 2) or merged blocks 0/2 (NBV 3);  Y = block 1
+    float bias_x[4], bias_y[4];   // log2-domain rpb, -inf outside the band
+    bool from0[4];                // NBV 3: slot r of X comes from block 0 (else block 2)
+    u32x2 keep0, keep2;           // NBV 3: 16-bit lane masks that split packed X into blocks 0 and 2
+};
+
+// `bias_lds` holds this head's rpb row times log2(e) in slots [0, W) (zeros without
+// rpb); it is filled by stage_bias() before the workgroup barrier.
+__device__ inline void stage_bias(LDS_PTR(float) bias_lds, const float *rpb_h, int W, int tid) {
+    if (tid < 32) bias_lds[tid] = (rpb_h && tid < W) ? rpb_h[tid] * kLog2e : 0.f;
+}
+__device__ inline float bias_at(LDS_PTR(float) bias_lds, int j, int W) {   // -inf outside the band
+    const float val = bias_lds[j & 31];
+    return (j >= 0 && j < W) ? val : kNegInf;
+}
+
+template <int NBV>
+__device__ inline void make_window(Window<NBV> &w, LDS_PTR(float) bias_lds, int W, int L, int shift, int g, int n) {
+    uint32_t m[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int j0 = 4 * g + r - shift - n + L;
+        w.bias_y[r] = bias_at(bias_lds, j0 + 16, W);
+        if (NBV == 2) {
+            w.from0[r] = true;
+            w.bias_x[r] = bias_at(bias_lds, j0, W);
+        } else {
+            w.from0[r] = j0 >= 0;
+            w.bias_x[r] = bias_at(bias_lds, w.from0[r] ? j0 : j0 + 32, W);
+        }
+        m[r] = w.from0[r] ? 0xffffu : 0u;
+    }
+    w.keep0 = u32x2{m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
+    w.keep2 = u32x2{~w.keep0.x, ~w.keep0.y};
+}
+
+// ---- work split ---------------------------------------------------------------
+struct Split {
+    int tiles;       // 16-row tiles per sequence
+    int nt;          // tiles per strip
+    int strips;      // strips per sequence
+    int64_t items;   // workgroups
+};
+inline Split make_split(int64_t B, int64_t T, int max_tiles) {
+    Split s;
+    s.tiles = (int)((T + 15) / 16);
+    s.strips = (s.tiles + max_tiles - 1) / max_tiles;
+    // small problems: more, shorter strips so that every CU gets a few workgroups
+    while (B * s.strips < 1024 && s.strips < s.tiles) ++s.strips;
+    s.nt = (s.tiles + s.strips - 1) / s.strips;
+    s.strips = (s.tiles + s.nt - 1) / s.nt;
+    s.items = B * s.strips;
+    return s;
+}
+
+// Workgroup id -> work item, so that consecutive items (neighbouring strips of a
+// sequence, which share halo rows) run on the same XCD and hit the same L2: the
+// hardware deals workgroup ids round-robin over the 8 XCDs.
+__device__ inline uint32_t xcd_item(uint32_t wg, uint32_t items) {
+    const uint32_t per = items / 8;          // items in the evenly dealt part
+    if (wg >= per * 8) return wg;            // ragged tail keeps its id
+    return (wg & 7) * per + (wg >> 3);
+}
+
+// Dynamic LDS above 64 KB has to be allowed per kernel.
+template <class K>
+inline bool allow_lds(K kern, size_t bytes) {
+    if (bytes <= 64 * 1024) return true;
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (int)bytes) == hipSuccess;
+}
+
+// Number of virtual key blocks the kernels need, 0 if the shape is not covered.
+inline int window_blocks(const Geom &g) {
+    const int R = g.W - 1 - g.L;
+    if (g.C != 16 && g.C != 32 && g.C != 64 && g.C != 128) return 0;
+    if (g.T > (1 << 29) / g.C) return 0;   // per-sequence byte offsets stay in 31 bits
+    if (15 + g.W <= 32) return 2;
+    if (g.L <= 16 && R <= 16 && g.W <= 32) return 3;
+    return 0;
+}
+
+#define NA1D_MFMA_DISPATCH(FN, ...)                                            \
+    do {                                                                       \
+        if (dtype == NA1D_BF16) {                                              \
+            switch (g.C) {                                                     \
+                case 16: return FN<BF16, 16>(__VA_ARGS__);                     \
+                case 32: return FN<BF16, 32>(__VA_ARGS__);                     \
+                case 64: return FN<BF16, 64>(__VA_ARGS__);                     \
+                case 128: return FN<BF16, 128>(__VA_ARGS__);                   \
+            }                                                                  \
+        } else {                                                               \
+            switch (g.C) {                                                     \
+                case 16: return FN<FP16, 16>(__VA_ARGS__);                     \
+                case 32: return FN<FP16, 32>(__VA_ARGS__);                     \
+                case 64: return FN<FP16, 64>(__VA_ARGS__);                     \
+                case 128: return FN<FP16, 128>(__VA_ARGS__);                   \
+            }                                                                  \
+        }                                                                      \
+        return NA1D_ERR_UNSUPPORTED;                                           \
+    } while (0)
+
+
+}  // namespace mfma
+}  // namespace na1d

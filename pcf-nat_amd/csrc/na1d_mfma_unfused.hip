@@ -1,0 +1,299 @@
+// The three un-fused NA1D primitives on the matrix cores (gfx950): band QK^T (P1),
+// band . V (P2) and the inverse-neighbourhood gather (P3), with the fp32 [B,T,W]
+// score tensor in memory as the reference's two-call API has it.  Tiling, LDS layout
+// and operand conventions are those of na1d_mfma_core.h; the score rows of a strip are
+// contiguous in memory (16*W floats per tile), so they move between HBM and LDS as
+// plain 16-byte copies and are picked apart / assembled per lane inside LDS.
+//
+// P2 and P3 round the scores to the 16-bit dtype before the contraction, as the
+// reference kernels do (bf16_ana1d_kernel.cu:305,414); accumulation is fp32.
+#include "na1d_mfma_core.h"
+
+namespace na1d {
+namespace mfma {
+
+// Copy `floats` fp32 values starting `first` floats into a sequence's score rows to LDS (or back),
+// 16 bytes per lane per round; the buffer resource zero-fills / drops what lies outside the sequence.
+// `first` is a multiple of 4 floats times 16 rows (a tile start), so units never straddle the start.
+constexpr int kMaxScoreRounds = (Strip<16>::kMaxTiles + 2) * 16 * 32 * 4 / 16 / kThreads;   // W <= 32
+
+struct ScoreStage {
+    u32x4 x[kMaxScoreRounds];
+    __device__ inline void issue(Rsrc src, int first, int tid) {
+#pragma unroll
+        for (int j = 0; j < kMaxScoreRounds; ++j)
+            x[j] = __builtin_amdgcn_raw_buffer_load_b128(src, (first + (j * kThreads + tid) * 4) * 4, 0, 0);
+    }
+    __device__ inline void commit(LDS_PTR(float) region, int floats, int tid) const {
+#pragma unroll
+        for (int j = 0; j < kMaxScoreRounds; ++j) {
+            const int u = j * kThreads + tid;
+            if (u * 4 < floats) *reinterpret_cast<LDS_PTR(u32x4)>(region + u * 4) = x[j];
+        }
+    }
+};
+
+__device__ inline float score_at(LDS_PTR(float) rows, int row, int j, int W) {   // 0 outside the band
+    const float val = rows[row * W + min(max(j, 0), W - 1)];
+    return (j >= 0 && j < W) ? val : 0.f;
+}
+
+// =============================================================================
+// P1: attn[b,t,j] = sum_c a[b,t,c] * b~[b,t-L+j,c]
+// =============================================================================
+template <class DT, int C, int NBV>
+__global__ void __launch_bounds__(kThreads)
+qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__restrict__ kb, uint32_t items, int T,
+          int W, int L, int tiles, int nt, int strips) {
+    using LL = Lds<C>;
+    constexpr int MT = Strip<C>::kMaxTiles;
+    // dynamic LDS: K region of nt+2 tiles, Q region of nt tiles, one 16 x W fp32 tile per wave
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) q_lds = k_lds + (nt + 2) * LL::kTileBytes;
+    LDS_PTR(float) out_lds = (LDS_PTR(float))(q_lds + nt * LL::kTileBytes);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = item / (uint32_t)strips;
+    const int strip = (int)(item - b * strips);
+    const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
+    const int g = lane >> 4, n = lane & 15;
+    const int shift = NBV == 3 ? 16 : L;
+
+    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    {
+        const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
+        Stage<C, MT + 2> sk;
+        Stage<C, MT> sq;
+        sk.issue(make_rsrc(kb + seq_off, key_bytes), 16 * i0 - 16, tid);
+        sq.issue(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, tid);
+        sk.commit(k_lds, nt + 2, tid);
+        sq.commit(q_lds, nt, tid);
+    }
+    const Rsrc as = make_rsrc(attn + (int64_t)b * T * W, T * W * 4);
+    RowLane<C> k_lane, q_lane;
+    k_lane.init(16 - shift, lane);
+    q_lane.init(0, lane);
+    LDS_PTR(float) mine = out_lds + wave * 16 * W;
+    __syncthreads();
+
+    for (int i = i0 + wave; i < i1; i += kWaves) {
+        const int tile_bytes = (i - i0) * LL::kTileBytes;
+        RowOperand<C> qt;
+        read_rows<C>(qt, q_lds + tile_bytes, q_lane);
+#pragma unroll
+        for (int vb = 0; vb < NBV; ++vb) {
+            RowOperand<C> kop;
+            read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
+            const f32x4 s = dot_rows_mma<DT, C>(kop, qt);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = 16 * vb + 4 * g + r - shift - n + L;
+                if (j >= 0 && j < W) mine[n * W + j] = s[r];      // every (row, slot) is written by exactly one lane
+            }
+        }
+        // LDS serves one wave's accesses in program order, so the other lanes' values are there when the
+        // reads below execute; the fence only keeps the compiler from moving them across
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const int first = 16 * i * W;                             // floats into the sequence's score rows
+        for (int u = lane; u * 4 < 16 * W; u += 64)
+            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, 0);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");    // tile read before the next one overwrites it
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+// =============================================================================
+// P2: out[b,t,c] = sum_j attn[b,t,j] * v~[b,t-L+j,c]
+// =============================================================================
+template <class DT, int C, int NBV>
+__global__ void __launch_bounds__(kThreads)
+av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ v, uint32_t items, int T,
+          int W, int L, int tiles, int nt, int strips) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16;
+    constexpr int MT = Strip<C>::kMaxTiles;
+    // dynamic LDS: V region of nt+2 tiles, score rows of the strip (nt*16 x W fp32)
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    LDS_PTR(char) v_lds = (LDS_PTR(char))smem;
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(v_lds + (nt + 2) * LL::kTileBytes);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = item / (uint32_t)strips;
+    const int strip = (int)(item - b * strips);
+    const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
+    const int g = lane >> 4, n = lane & 15;
+    const int shift = NBV == 3 ? 16 : L;
+
+    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    {
+        const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C;
+        Stage<C, MT + 2> sv;
+        ScoreStage ss;
+        sv.issue(make_rsrc(v + seq_off, key_bytes), 16 * i0 - 16, tid);
+        ss.issue(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, tid);
+        sv.commit(v_lds, nt + 2, tid);
+        ss.commit(s_lds, nt * 16 * W, tid);
+    }
+    const Rsrc os = make_rsrc(out + seq_off, T * 2 * C);
+    TrLane<C> v_lane;
+    v_lane.init(16 - shift, lane);
+    __syncthreads();
+
+    for (int i = i0 + wave; i < i1; i += kWaves) {
+        const int tile_bytes = (i - i0) * LL::kTileBytes;
+        LDS_PTR(float) rows = s_lds + (i - i0) * 16 * W;
+        f32x4 o[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int vb = 0; vb < NBV; ++vb) {
+            float p[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) p[r] = score_at(rows, n, 16 * vb + 4 * g + r - shift - n + L, W);
+            const u32x2 pb = {Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+            LDS_PTR(char) blk = v_lds + tile_bytes + vb * LL::kTileBytes;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr(blk + v_lane.off[ct]), pb, o[ct]);
+        }
+        const int qrow = 16 * i + n;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            u32x2 w;
+            w.x = Mma<DT>::pack(o[ct][0], o[ct][1]);
+            w.y = Mma<DT>::pack(o[ct][2], o[ct][3]);
+            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * (2 * C) + ct * 32 + g * 8, 0, 0);
+        }
+    }
+}
+
+// =============================================================================
+// P3: out[b,u,c] = sum_j attn[b,u+L-j,j] * x[b,u+L-j,c]
+// =============================================================================
+template <class DT, int C, int NBV>
+__global__ void __launch_bounds__(kThreads)
+gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ x, uint32_t items,
+              int T, int W, int L, int tiles, int nt, int strips) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16;
+    constexpr int MT = Strip<C>::kMaxTiles;
+    // dynamic LDS: x rows of query tiles i0-1 .. i1 (nt+2 tiles) and their score rows ((nt+2)*16 x W fp32)
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    LDS_PTR(char) x_lds = (LDS_PTR(char))smem;
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + (nt + 2) * LL::kTileBytes);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = item / (uint32_t)strips;
+    const int strip = (int)(item - b * strips);
+    const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
+    const int g = lane >> 4, n = lane & 15;
+    const int shift = NBV == 3 ? 16 : L;
+
+    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    {
+        const int rows_hi = min(T, 16 * (i1 + 1));
+        Stage<C, MT + 2> sx;
+        ScoreStage ss;
+        sx.issue(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * i0 - 16, tid);
+        ss.issue(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), (16 * i0 - 16) * W, tid);
+        sx.commit(x_lds, nt + 2, tid);
+        ss.commit(s_lds, (nt + 2) * 16 * W, tid);
+    }
+    TrLane<C> x_tr;
+    x_tr.init(0, lane);
+    const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
+    const Rsrc os = make_rsrc(out + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
+    __syncthreads();
+
+    // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb; lane (n, g)
+    // holds key row n of the block against queries 4g+r of that tile: slot j = 16*vb - shift + n - (4g+r) + L
+    const int kp_lo = i0 + (shift == 16 ? 1 : 0), kp_hi = i1 - (shift == 0 ? 1 : 0);
+    for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
+        f32x4 acc[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int vb = 0; vb < NBV; ++vb) {
+            const int tq = kp - vb - (i0 - 1);
+            LDS_PTR(float) rows = s_lds + tq * 16 * W;
+            float p[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) p[r] = score_at(rows, 4 * g + r, 16 * vb - shift + n - (4 * g + r) + L, W);
+            const u32x2 pb = {Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+            LDS_PTR(char) xt = x_lds + tq * LL::kTileBytes;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(xt + x_tr.off[ct]), pb, acc[ct]);
+        }
+        const int row_off = (16 * (kp - i0) - shift + n) * (2 * C);     // outside the strip -> dropped
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            u32x2 w;
+            w.x = Mma<DT>::pack(acc[ct][0], acc[ct][1]);
+            w.y = Mma<DT>::pack(acc[ct][2], acc[ct][3]);
+            __builtin_amdgcn_raw_buffer_store_b64(w, os, row_off + ct * 32 + g * 8, 0, 0);
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------- launchers
+template <class DT, int C>
+int launch_qk(float *attn, const void *a, const void *b, const Geom &g, hipStream_t s) {
+    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
+    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    auto kern = window_blocks(g) == 2 ? qk_kernel<DT, C, 2> : qk_kernel<DT, C, 3>;
+    const size_t lds = (size_t)(2 * sp.nt + 2) * Lds<C>::kTileBytes + (size_t)kWaves * 16 * g.W * sizeof(float);
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>(attn, (const char *)a, (const char *)b, (uint32_t)sp.items,
+                                                   (int)g.T, g.W, g.L, sp.tiles, sp.nt, sp.strips);
+    return launch_status();
+}
+
+template <class DT, int C>
+int launch_av(void *out, const float *attn, const void *v, const Geom &g, hipStream_t s) {
+    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
+    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    auto kern = window_blocks(g) == 2 ? av_kernel<DT, C, 2> : av_kernel<DT, C, 3>;
+    const size_t lds = (size_t)(sp.nt + 2) * Lds<C>::kTileBytes + (size_t)sp.nt * 16 * g.W * sizeof(float) + 16;
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)v, (uint32_t)sp.items, (int)g.T,
+                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips);
+    return launch_status();
+}
+
+template <class DT, int C>
+int launch_gather(void *out, const float *attn, const void *x, const Geom &g, hipStream_t s) {
+    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
+    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    auto kern = window_blocks(g) == 2 ? gather_kernel<DT, C, 2> : gather_kernel<DT, C, 3>;
+    const size_t lds = (size_t)(sp.nt + 2) * Lds<C>::kTileBytes + (size_t)(sp.nt + 2) * 16 * g.W * sizeof(float) + 16;
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)x, (uint32_t)sp.items, (int)g.T,
+                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips);
+    return launch_status();
+}
+
+// The score tensor is addressed with 32-bit byte offsets inside a sequence.
+inline bool scores_fit(const Geom &g) { return g.T <= (1 << 29) / (4 * g.W); }
+
+int qk(float *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s) {
+    if (!window_blocks(g) || !scores_fit(g)) return NA1D_ERR_UNSUPPORTED;
+    NA1D_MFMA_DISPATCH(launch_qk, attn, a, b, g, s);
+}
+int av(void *out, const float *attn, const void *v, const Geom &g, int dtype, hipStream_t s) {
+    if (!window_blocks(g) || !scores_fit(g)) return NA1D_ERR_UNSUPPORTED;
+    NA1D_MFMA_DISPATCH(launch_av, out, attn, v, g, s);
+}
+int gather(void *out, const float *attn, const void *x, const Geom &g, int dtype, hipStream_t s) {
+    if (!window_blocks(g) || !scores_fit(g)) return NA1D_ERR_UNSUPPORTED;
+    NA1D_MFMA_DISPATCH(launch_gather, out, attn, x, g, s);
+}
+
+}  // namespace mfma
+}  // namespace na1d

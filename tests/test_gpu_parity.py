@@ -265,6 +265,39 @@ def test_deterministic_rpb_gradient_is_bit_reproducible():
     assert torch.allclose(grads[0][0], grads[2][0], rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_two_kernel_families_agree(dtype):
+    """The matrix-core kernels and the generic kernels are independent implementations; NA1D_FORCE_GENERIC=1
+    routes the same C-ABI calls to the generic ones."""
+    N, H, T, C, W, L = 3, 4, 150, 32, 15, 7
+    B = N * H
+    q, k, v, do = dev(*make_inputs(B, T, C, W, 81, dtype, n=4, scale=C ** -0.5))
+    s = seeded_scores(B, T, W, 9).cuda()
+    rpb = (torch.randn(H, W, generator=torch.Generator().manual_seed(6)) * 0.3).cuda()
+    tv = torch.tensor([T, T - 17, 40], dtype=torch.int32).cuda()
+
+    def run_all():
+        attn = _unfused("na1d_qk_forward", torch.empty(B, T, W, device="cuda"), q, k, W, L)
+        av = _unfused("na1d_av_forward", torch.empty_like(v), s, v, W, L)
+        ga = _unfused("na1d_k_backward", torch.empty_like(q), s, q, W, L)
+        qd, kd, vd = (t.clone().requires_grad_(True) for t in (q, k, v))
+        rd = rpb.clone().requires_grad_(True)
+        o = na1d_fused(qd, kd, vd, W, L, rpb=rd, t_valid=tv, num_heads=H)
+        o.backward(do)
+        return [attn, av.float(), ga.float(), o.detach().float(), qd.grad.float(), kd.grad.float(), vd.grad.float(), rd.grad]
+
+    fast = run_all()
+    os.environ["NA1D_FORCE_GENERIC"] = "1"
+    try:
+        slow = run_all()
+    finally:
+        del os.environ["NA1D_FORCE_GENERIC"]
+    assert O.rel_l2(fast[0], slow[0]) < 1e-5
+    for a, b in zip(fast[1:], slow[1:]):
+        assert O.rel_l2(a, b) < TOL[dtype]
+    assert not torch.equal(fast[1], slow[1]) or not torch.equal(fast[3], slow[3])     # they really are different code
+
+
 def test_runs_on_the_current_stream():
     """Launches go to torch's current stream (the reference uses the legacy default
     stream; its data prefetcher runs a side stream, public/Utils.py:89-100)."""
