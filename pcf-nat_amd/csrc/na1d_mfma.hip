@@ -13,24 +13,25 @@ __global__ void __launch_bounds__(kThreads)
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
-                 int strips, float scale) {
+                 int strips, float scale, uint32_t strips_magic, uint32_t heads_magic) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = Strip<C>::kMaxTiles;
+    fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic);
     // dynamic LDS (fwd_lds_bytes): K and V regions of nt+2 tiles, Q region of nt tiles, 32 bias floats
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int key_region = (nt + 2) * LL::kTileBytes;
+    const int key_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
     LDS_PTR(char) q_lds = v_lds + key_region;
-    LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + nt * LL::kTileBytes);
+    LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + region_bytes<C>(nt));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t item = xcd_item(blockIdx.x, items);
-    const uint32_t b = item / (uint32_t)strips;
+    const uint32_t b = div_by(item, strips, strips_magic);
     const int strip = (int)(item - b * strips);
-    const uint32_t sample = b / (uint32_t)H, head = b - sample * H;
+    const uint32_t sample = div_by(b, H, heads_magic), head = b - sample * H;
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
     const int shift = NBV == 3 ? 16 : L;
@@ -46,15 +47,11 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
 
     // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
     {
-        Stage<C, MT + 2> sk, sv;
-        Stage<C, MT> sq;
-        sk.issue(ks, 16 * i0 - 16, tid);
-        sv.issue(vs, 16 * i0 - 16, tid);
-        sq.issue(qs, 16 * i0, tid);
+        const int lane_off = direct_lane_offset<C>(wave, lane);
+        stage_direct<C, MT + 2>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off);
+        stage_direct<C, MT>(qs, 16 * i0, q_lds, nt, wave, lane_off);
+        stage_direct<C, MT + 2>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off);
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
-        sk.commit(k_lds, nt + 2, tid);
-        sv.commit(v_lds, nt + 2, tid);
-        sq.commit(q_lds, nt, tid);
     }
 
     int tv = T;
@@ -68,6 +65,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     q_lane.init(0, lane);
     v_lane.init(16 - shift, lane);
 
+    wait_direct();
     __syncthreads();
     Window<NBV> win;
     make_window<NBV>(win, bias_lds, W, L, shift, g, n);
@@ -159,13 +157,13 @@ template <class DT, int C>
 int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
                const int32_t *t_valid, const Geom &g, float scale, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips) || !div_magic_ok(g.B, g.H)) return NA1D_ERR_UNSUPPORTED;
     auto kern = window_blocks(g) == 2 ? fused_fwd_kernel<DT, C, 2> : fused_fwd_kernel<DT, C, 3>;
-    const size_t lds = (size_t)(3 * sp.nt + 4) * Lds<C>::kTileBytes + 32 * sizeof(float);
+    const size_t lds = (size_t)2 * region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt) + 32 * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                                                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
-                                                 sp.nt, sp.strips, scale);
+                                                 sp.nt, sp.strips, scale, div_magic(sp.strips), div_magic(g.H));
     return launch_status();
 }
 
@@ -214,7 +212,11 @@ drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, 
 }
 
 template <int C> struct StripBwd {
+#ifdef NA1D_BWD_MT
+    static constexpr int kMaxTiles = NA1D_BWD_MT * 32 / (C < 32 ? 32 : C);
+#else
     static constexpr int kMaxTiles = C <= 32 ? 8 : C <= 64 ? 4 : 2;
+#endif
 };
 
 template <class DT, int C, int NBV>
@@ -223,36 +225,39 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
-                 int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes) {
+                 int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes, uint32_t strips_magic,
+                 uint32_t heads_magic) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
+    fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
+                   drpb_partial, kv_bytes, strips_magic, heads_magic);
     constexpr int kRowsQ = (MT + 2) * 16;
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
-    static_assert(kRowsQ <= kThreads, "one thread per staged lse row");
+    static_assert(kRowsQ <= kThreads, "one lane per staged lse row");
     // dynamic LDS (see launch_bwd): [K region | V region] of nt+4 tiles each (rows 16*i0 - 32 ...), reused after
     // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt+2 tiles (rows 16*i0 - 16 ...); lse
     // of the query-side rows; 32 bias floats; and - only when d rpb is wanted - per-lane partial sums and 8
     // partial sums per slot
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int key_region = (nt + 4) * LL::kTileBytes, qry_region = (nt + 2) * LL::kTileBytes;
+    const int key_region = region_bytes<C>(nt + 4), qry_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
     LDS_PTR(char) sc_lds = k_lds;                  // score tiles [(tq*2 + X/Y)*2 + P/dS]
     LDS_PTR(char) q_lds = k_lds + kv_bytes;
     LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
     LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
-    LDS_PTR(float) bias_lds = lse_lds + kRowsQ;
+    LDS_PTR(float) bias_lds = lse_lds + kThreads;
     LDS_PTR(float) rpart = bias_lds + 32;          // [kWaves * 8][64]
     LDS_PTR(float) rsum = rpart + kWaves * 8 * 64; // [8][32]
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t item = xcd_item(blockIdx.x, items);
-    const uint32_t b = item / (uint32_t)strips;
+    const uint32_t b = div_by(item, strips, strips_magic);
     const int strip = (int)(item - b * strips);
-    const uint32_t sample = b / (uint32_t)H, head = b - sample * H;
+    const uint32_t sample = div_by(b, H, heads_magic), head = b - sample * H;
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
     const int shift = NBV == 3 ? 16 : L;
@@ -264,20 +269,14 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         const Rsrc ks = make_rsrc(k + seq_off, key_bytes), vs = make_rsrc(v + seq_off, key_bytes);
         const Rsrc qs = make_rsrc(q + seq_off, qry_bytes), gs = make_rsrc(dout + seq_off, qry_bytes);
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
-        Stage<C, MT + 4> sk, sv;
-        Stage<C, MT + 2> sq, sg;
-        sk.issue(ks, 16 * i0 - 32, tid);
-        sv.issue(vs, 16 * i0 - 32, tid);
-        sq.issue(qs, 16 * i0 - 16, tid);
-        sg.issue(gs, 16 * i0 - 16, tid);
-        float l = 0.f;
-        if (tid < kRowsQ) l = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ls, (16 * i0 - 16 + tid) * 4, 0, 0));
+        const int lane_off = direct_lane_offset<C>(wave, lane);
+        // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * i0 - 16 + tid) * 4, 0, 0, 0);
+        stage_direct<C, MT + 4>(ks, 16 * i0 - 32, k_lds, nt + 4, wave, lane_off);
+        stage_direct<C, MT + 2>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off);
+        stage_direct<C, MT + 4>(vs, 16 * i0 - 32, v_lds, nt + 4, wave, lane_off);
+        stage_direct<C, MT + 2>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off);
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
-        sk.commit(k_lds, nt + 4, tid);
-        sv.commit(v_lds, nt + 4, tid);
-        sq.commit(q_lds, nt + 2, tid);
-        sg.commit(g_lds, nt + 2, tid);
-        if (tid < kRowsQ) lse_lds[tid] = l * kLog2e;
     }
 
     int tv = T;
@@ -292,6 +291,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     qry_lane.init(0, lane);
     qry_tr.init(0, lane);
 
+    wait_direct();
     __syncthreads();
     Window<NBV> win;
     make_window<NBV>(win, bias_lds, W, L, shift, g, n);
@@ -319,7 +319,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             s[vb] = dot_rows_mma<DT, C>(kop, qop);
             dp[vb] = dot_rows_mma<DT, C>(vop, gop);
         }
-        const float lse2 = lse_lds[tq * 16 + n];
+        const float lse2 = lse_lds[tq * 16 + n] * kLog2e;
         float zx[4], zy[4], dpx[4], dpy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -432,6 +432,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
         rsum[p * 32 + j] = sum;
     }
+    
     __syncthreads();
 
     // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
@@ -504,20 +505,21 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                const void *dout, const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g,
                float scale, float *workspace, int64_t workspace_bytes, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, StripBwd<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips) || !div_magic_ok(g.B, g.H)) return NA1D_ERR_UNSUPPORTED;
     float *partial = nullptr;
     if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
     auto kern = window_blocks(g) == 2 ? fused_bwd_kernel<DT, C, 2> : fused_bwd_kernel<DT, C, 3>;
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
-    const int kv_bytes = std::max(2 * (sp.nt + 4) * Lds<C>::kTileBytes, (sp.nt + 2) * 4 * 512);
-    const size_t lds = (size_t)kv_bytes + (size_t)2 * (sp.nt + 2) * Lds<C>::kTileBytes +
-                       ((StripBwd<C>::kMaxTiles + 2) * 16 + 32 + (drpb ? kWaves * 8 * 64 + 8 * 32 : 0)) * sizeof(float);
+    const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 4), (sp.nt + 2) * 4 * 512);
+    const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
+                       (kThreads + 32 + (drpb ? kWaves * 8 * 64 + 8 * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                                                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
                                                  t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
-                                                 sp.nt, sp.strips, scale, partial, kv_bytes);
-    if (partial)
+                                                 sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
+                                                 div_magic(g.H));
+    if (partial && drpb)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();
 }

@@ -31,9 +31,9 @@
 // Work.  A workgroup of four waves owns a strip of up to kMaxTiles<C> consecutive
 // tiles of one sequence.  It first copies the strip's rows of every operand
 // (plus one 16-row halo block each side for the key-side operands) into LDS with
-// all loads in flight at once - buffer loads, so rows outside the sequence read
-// as zero, which is the band's zero fill - then, after one barrier, each wave
-// computes tiles wave, wave+4, ... entirely out of LDS.
+// all loads in flight at once - buffer loads that write LDS directly, so rows
+// outside the sequence arrive as zeros, which is the band's zero fill - then, after
+// one barrier, each wave computes tiles wave, wave+4, ... entirely out of LDS.
 #pragma once
 
 #include <algorithm>
@@ -116,34 +116,47 @@ template <int C> struct Lds {
 
 // Tiles per strip (compile-time ceiling that sizes LDS and the copy loops).
 template <int C> struct Strip {
+#ifdef NA1D_FWD_MT
+    static constexpr int kMaxTiles = NA1D_FWD_MT * 32 / (C < 32 ? 32 : C);
+#else
     static constexpr int kMaxTiles = C <= 16 ? 8 : C <= 32 ? 8 : C <= 64 ? 4 : 2;
+#endif
 };
 
 // Copy up to NTILES tiles of rows, starting at row_lo of a sequence, into an LDS
-// region, all loads in flight before the first LDS store.  Split in two so several
-// regions' loads can be issued back to back.  NTILES fixes the (unrolled) number of
-// loads per thread; the caller's buffer resource ends where the wanted rows end, so
-// surplus loads fetch nothing.
-template <int C, int NTILES> struct Stage {
-    static constexpr int kTotal = NTILES * 16 * Lds<C>::kUnits;             // 16-byte units
-    static constexpr int kRounds = (kTotal + kThreads - 1) / kThreads;
-    u32x4 x[kRounds];
-    __device__ inline void issue(Rsrc src, int row_lo, int tid) {
+// region with buffer loads that write LDS directly: no registers are held while the
+// loads are in flight.  NTILES fixes the (unrolled) number of loads per wave; the
+// caller's buffer resource ends where the wanted rows end.  One wave's
+// load fills 1 KB of consecutive LDS (lane l -> bytes 16l .. 16l+15 behind the
+// wave-uniform base), so each lane asks for the 16-byte unit that belongs at that
+// place under the XOR swizzle.  Chunk c of a region is loaded by wave c % kWaves; the
+// swizzle repeats every four chunks at most, so a lane's offset inside its chunk is
+// one constant.  Regions are padded to whole chunks (region_bytes); rows outside the
+// resource arrive as zeros.  The loads count on vmcnt: wait for them before the
+// workgroup barrier that publishes the regions.
+constexpr int kChunk = 1024;
+static_assert(kWaves % 4 == 0, "chunk -> swizzle phase mapping assumes a multiple of four waves");
+template <int C> constexpr int region_bytes(int ntiles) {
+    return (ntiles * Lds<C>::kTileBytes + kChunk - 1) / kChunk * kChunk;
+}
+template <int C> __device__ inline int direct_lane_offset(int wave, int lane) {
+    const int u = wave * 64 + lane;      // 16-byte unit inside chunks wave, wave + 4, ...
+    const int su = u % Lds<C>::kUnits;
+    return (lane - su + (su ^ Lds<C>::swz(u / Lds<C>::kUnits))) * 16;
+}
+template <int C, int NTILES>
+__device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, int ntiles, int wave, int lane_off) {
+    constexpr int kRounds = (region_bytes<C>(NTILES) / kChunk + kWaves - 1) / kWaves;
+    const int chunks = region_bytes<C>(ntiles) / kChunk;
+    const int base = row_lo * Lds<C>::kRowBytes + lane_off;
 #pragma unroll
-        for (int j = 0; j < kRounds; ++j)
-            x[j] = __builtin_amdgcn_raw_buffer_load_b128(src, (row_lo * Lds<C>::kUnits + j * kThreads + tid) * 16, 0, 0);
+    for (int j = 0; j < kRounds; ++j) {
+        const int c = j * kWaves + wave;
+        if (c < chunks)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * kChunk), 16, base + c * kChunk, 0, 0, 0);
     }
-    // `ntiles` <= NTILES: the region only has room for that many tiles
-    __device__ inline void commit(LDS_PTR(char) region, int ntiles, int tid) const {
-        const int total = ntiles * 16 * Lds<C>::kUnits;
-#pragma unroll
-        for (int j = 0; j < kRounds; ++j) {
-            const int u = j * kThreads + tid;
-            if (u < total)
-                *reinterpret_cast<LDS_PTR(u32x4)>(region + Lds<C>::addr(u / Lds<C>::kUnits, (u % Lds<C>::kUnits) * 16)) = x[j];
-        }
-    }
-};
+}
+__device__ inline void wait_direct() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // ---- operands out of LDS ------------------------------------------------------
 // Row operand (A or B of a contraction over channels): lane (n, g) holds row n of a
@@ -270,7 +283,21 @@ __device__ inline void make_window(Window<NBV> &w, LDS_PTR(float) bias_lds, int 
     w.keep2 = u32x2{~w.keep0.x, ~w.keep0.y};
 }
 
+// Kernel arguments live in memory and the compiler fetches each one next to its
+// first use, which here puts a scalar-load round trip in front of every region's
+// copy.  Naming them in an empty asm at kernel entry makes all the fetches go out
+// together, behind one wait.
+template <class... A> __device__ inline void fetch_args_now(A... a) {
+    ((void)0, ..., [](auto x) { asm volatile("" ::"s"(x)); }(a));
+}
+
 // ---- work split ---------------------------------------------------------------
+// Division of a wave-uniform number by a launch constant d as one multiply-high:
+// with m = floor(2^32 / d) + 1 the quotient is exact whenever n * d < 2^32.
+inline uint32_t div_magic(int64_t d) { return d > 1 ? (uint32_t)((1ull << 32) / (uint64_t)d) + 1u : 0u; }
+inline bool div_magic_ok(int64_t n_max, int64_t d) { return n_max < (1ll << 32) / d; }
+__device__ inline uint32_t div_by(uint32_t n, int d, uint32_t magic) { return d == 1 ? n : __umulhi(n, magic); }
+
 struct Split {
     int tiles;       // 16-row tiles per sequence
     int nt;          // tiles per strip

@@ -12,26 +12,23 @@
 namespace na1d {
 namespace mfma {
 
-// Copy `floats` fp32 values starting `first` floats into a sequence's score rows to LDS (or back),
-// 16 bytes per lane per round; the buffer resource zero-fills / drops what lies outside the sequence.
-// `first` is a multiple of 4 floats times 16 rows (a tile start), so units never straddle the start.
-constexpr int kMaxScoreRounds = (Strip<16>::kMaxTiles + 2) * 16 * 32 * 4 / 16 / kThreads;   // W <= 32
-
-struct ScoreStage {
-    u32x4 x[kMaxScoreRounds];
-    __device__ inline void issue(Rsrc src, int first, int tid) {
+// Copy `floats` fp32 values starting `first` floats into a sequence's score rows straight into LDS, one
+// 1 KB chunk per wave and round (see stage_direct); the buffer resource zero-fills what lies outside the
+// rows the strip needs.  `first` is a tile start, so 16-byte units never straddle the sequence's start.
+// The region is padded to whole chunks (score_bytes).
+inline __host__ __device__ int score_bytes(int tiles, int W) { return (tiles * 16 * W * 4 + kChunk - 1) / kChunk * kChunk; }
+template <int C>
+__device__ inline void stage_scores(Rsrc src, int first, LDS_PTR(float) region, int tiles, int W, int wave, int lane) {
+    constexpr int kRounds = ((Strip<C>::kMaxTiles + 2) * 16 * 32 * 4 / kChunk + kWaves - 1) / kWaves;   // W <= 32
+    const int chunks = score_bytes(tiles, W) / kChunk;
 #pragma unroll
-        for (int j = 0; j < kMaxScoreRounds; ++j)
-            x[j] = __builtin_amdgcn_raw_buffer_load_b128(src, (first + (j * kThreads + tid) * 4) * 4, 0, 0);
+    for (int j = 0; j < kRounds; ++j) {
+        const int c = j * kWaves + wave;
+        if (c < chunks)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * (kChunk / 4)), 16,
+                                                     first * 4 + c * kChunk + lane * 16, 0, 0, 0);
     }
-    __device__ inline void commit(LDS_PTR(float) region, int floats, int tid) const {
-#pragma unroll
-        for (int j = 0; j < kMaxScoreRounds; ++j) {
-            const int u = j * kThreads + tid;
-            if (u * 4 < floats) *reinterpret_cast<LDS_PTR(u32x4)>(region + u * 4) = x[j];
-        }
-    }
-};
+}
 
 __device__ inline float score_at(LDS_PTR(float) rows, int row, int j, int W) {   // 0 outside the band
     const float val = rows[row * W + min(max(j, 0), W - 1)];
@@ -44,19 +41,20 @@ __device__ inline float score_at(LDS_PTR(float) rows, int row, int j, int W) {  
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__restrict__ kb, uint32_t items, int T,
-          int W, int L, int tiles, int nt, int strips) {
+          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic) {
     using LL = Lds<C>;
     constexpr int MT = Strip<C>::kMaxTiles;
+    fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic);
     // dynamic LDS: K region of nt+2 tiles, Q region of nt tiles, one 16 x W fp32 tile per wave
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) q_lds = k_lds + (nt + 2) * LL::kTileBytes;
-    LDS_PTR(float) out_lds = (LDS_PTR(float))(q_lds + nt * LL::kTileBytes);
+    LDS_PTR(char) q_lds = k_lds + region_bytes<C>(nt + 2);
+    LDS_PTR(float) out_lds = (LDS_PTR(float))(q_lds + region_bytes<C>(nt));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t item = xcd_item(blockIdx.x, items);
-    const uint32_t b = item / (uint32_t)strips;
+    const uint32_t b = div_by(item, strips, strips_magic);
     const int strip = (int)(item - b * strips);
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
@@ -65,18 +63,16 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
         const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
-        Stage<C, MT + 2> sk;
-        Stage<C, MT> sq;
-        sk.issue(make_rsrc(kb + seq_off, key_bytes), 16 * i0 - 16, tid);
-        sq.issue(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, tid);
-        sk.commit(k_lds, nt + 2, tid);
-        sq.commit(q_lds, nt, tid);
+        const int lane_off = direct_lane_offset<C>(wave, lane);
+        stage_direct<C, MT + 2>(make_rsrc(kb + seq_off, key_bytes), 16 * i0 - 16, k_lds, nt + 2, wave, lane_off);
+        stage_direct<C, MT>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off);
     }
     const Rsrc as = make_rsrc(attn + (int64_t)b * T * W, T * W * 4);
     RowLane<C> k_lane, q_lane;
     k_lane.init(16 - shift, lane);
     q_lane.init(0, lane);
     LDS_PTR(float) mine = out_lds + wave * 16 * W;
+    wait_direct();
     __syncthreads();
 
     for (int i = i0 + wave; i < i1; i += kWaves) {
@@ -112,19 +108,20 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ v, uint32_t items, int T,
-          int W, int L, int tiles, int nt, int strips) {
+          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = Strip<C>::kMaxTiles;
+    fetch_args_now(out, attn, v, items, T, W, L, tiles, nt, strips, strips_magic);
     // dynamic LDS: V region of nt+2 tiles, score rows of the strip (nt*16 x W fp32)
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) v_lds = (LDS_PTR(char))smem;
-    LDS_PTR(float) s_lds = (LDS_PTR(float))(v_lds + (nt + 2) * LL::kTileBytes);
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(v_lds + region_bytes<C>(nt + 2));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t item = xcd_item(blockIdx.x, items);
-    const uint32_t b = item / (uint32_t)strips;
+    const uint32_t b = div_by(item, strips, strips_magic);
     const int strip = (int)(item - b * strips);
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
@@ -133,16 +130,14 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
         const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C;
-        Stage<C, MT + 2> sv;
-        ScoreStage ss;
-        sv.issue(make_rsrc(v + seq_off, key_bytes), 16 * i0 - 16, tid);
-        ss.issue(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, tid);
-        sv.commit(v_lds, nt + 2, tid);
-        ss.commit(s_lds, nt * 16 * W, tid);
+        stage_direct<C, MT + 2>(make_rsrc(v + seq_off, key_bytes), 16 * i0 - 16, v_lds, nt + 2, wave,
+                                direct_lane_offset<C>(wave, lane));
+        stage_scores<C>(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, s_lds, nt, W, wave, lane);
     }
     const Rsrc os = make_rsrc(out + seq_off, T * 2 * C);
     TrLane<C> v_lane;
     v_lane.init(16 - shift, lane);
+    wait_direct();
     __syncthreads();
 
     for (int i = i0 + wave; i < i1; i += kWaves) {
@@ -178,19 +173,20 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ x, uint32_t items,
-              int T, int W, int L, int tiles, int nt, int strips) {
+              int T, int W, int L, int tiles, int nt, int strips, uint32_t strips_magic) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = Strip<C>::kMaxTiles;
+    fetch_args_now(out, attn, x, items, T, W, L, tiles, nt, strips, strips_magic);
     // dynamic LDS: x rows of query tiles i0-1 .. i1 (nt+2 tiles) and their score rows ((nt+2)*16 x W fp32)
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) x_lds = (LDS_PTR(char))smem;
-    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + (nt + 2) * LL::kTileBytes);
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + region_bytes<C>(nt + 2));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t item = xcd_item(blockIdx.x, items);
-    const uint32_t b = item / (uint32_t)strips;
+    const uint32_t b = div_by(item, strips, strips_magic);
     const int strip = (int)(item - b * strips);
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
@@ -199,17 +195,15 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
         const int rows_hi = min(T, 16 * (i1 + 1));
-        Stage<C, MT + 2> sx;
-        ScoreStage ss;
-        sx.issue(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * i0 - 16, tid);
-        ss.issue(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), (16 * i0 - 16) * W, tid);
-        sx.commit(x_lds, nt + 2, tid);
-        ss.commit(s_lds, (nt + 2) * 16 * W, tid);
+        stage_direct<C, MT + 2>(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * i0 - 16, x_lds, nt + 2, wave,
+                                direct_lane_offset<C>(wave, lane));
+        stage_scores<C>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), (16 * i0 - 16) * W, s_lds, nt + 2, W, wave, lane);
     }
     TrLane<C> x_tr;
     x_tr.init(0, lane);
     const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
     const Rsrc os = make_rsrc(out + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
+    wait_direct();
     __syncthreads();
 
     // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb; lane (n, g)
@@ -246,36 +240,36 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
 template <class DT, int C>
 int launch_qk(float *attn, const void *a, const void *b, const Geom &g, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
     auto kern = window_blocks(g) == 2 ? qk_kernel<DT, C, 2> : qk_kernel<DT, C, 3>;
-    const size_t lds = (size_t)(2 * sp.nt + 2) * Lds<C>::kTileBytes + (size_t)kWaves * 16 * g.W * sizeof(float);
+    const size_t lds = (size_t)region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt) + (size_t)kWaves * 16 * g.W * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>(attn, (const char *)a, (const char *)b, (uint32_t)sp.items,
-                                                   (int)g.T, g.W, g.L, sp.tiles, sp.nt, sp.strips);
+                                                   (int)g.T, g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips));
     return launch_status();
 }
 
 template <class DT, int C>
 int launch_av(void *out, const float *attn, const void *v, const Geom &g, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
     auto kern = window_blocks(g) == 2 ? av_kernel<DT, C, 2> : av_kernel<DT, C, 3>;
-    const size_t lds = (size_t)(sp.nt + 2) * Lds<C>::kTileBytes + (size_t)sp.nt * 16 * g.W * sizeof(float) + 16;
+    const size_t lds = (size_t)region_bytes<C>(sp.nt + 2) + score_bytes(sp.nt, g.W);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)v, (uint32_t)sp.items, (int)g.T,
-                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips);
+                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips));
     return launch_status();
 }
 
 template <class DT, int C>
 int launch_gather(void *out, const float *attn, const void *x, const Geom &g, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL) return NA1D_ERR_UNSUPPORTED;
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
     auto kern = window_blocks(g) == 2 ? gather_kernel<DT, C, 2> : gather_kernel<DT, C, 3>;
-    const size_t lds = (size_t)(sp.nt + 2) * Lds<C>::kTileBytes + (size_t)(sp.nt + 2) * 16 * g.W * sizeof(float) + 16;
+    const size_t lds = (size_t)region_bytes<C>(sp.nt + 2) + score_bytes(sp.nt + 2, g.W);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)x, (uint32_t)sp.items, (int)g.T,
-                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips);
+                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips));
     return launch_status();
 }
 
