@@ -128,6 +128,43 @@ int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb,
                         int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
                         float scale, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
 
+/*
+ * The same two operators on strided tensors.  They have no counterpart among the
+ * reference's six native functions: they replace, together with the fused operator,
+ * the head split / merge copies around it (models/PCF_NATransformer.py:126-139,
+ * 151-152; models/MFA_NATransformer.py:127-138,150-151) by reading q, k, v straight
+ * out of the qkv projection's output and writing `out` straight into the layout the
+ * output projection reads.
+ *
+ *   N, H        : samples and heads (the packed entry points' B is N * H)
+ *   qkv_strides : int64[3] = {sample, head, row} strides, in elements, shared by q, k, v
+ *                 (and dq, dk, dv); element (n, h, t, c) of q is q[n*sample + h*head +
+ *                 t*row + c].  E.g. for a projection output [N, T, 3, H, C]:
+ *                 q = base, k = base + H*C, v = base + 2*H*C, strides {T*3*H*C, C, 3*H*C}.
+ *   out_strides : the same for out (and dout); [N, T, H*C] is {T*H*C, C, H*C}.
+ *   lse         : fp32 [N*H, T], packed
+ * Strides must be multiples of 8 elements and row >= C; the caller guarantees that
+ * distinct (n, h, t) rows do not overlap.  Returns NA1D_ERR_UNSUPPORTED when no
+ * matrix-core kernel covers the shape (C not in {16, 32, 64, 128}, W > 32, or more
+ * than 16 keys on one side): the caller then packs the tensors and uses the packed
+ * entry points.  The backward needs no `out`.
+ */
+int na1d_fused_forward_strided(void *out, float *lse,
+                               const void *q, const void *k, const void *v,
+                               const float *rpb, const int32_t *t_valid,
+                               int64_t N, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
+                               float scale, int dtype,
+                               const int64_t *qkv_strides, const int64_t *out_strides, void *stream);
+
+int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb,
+                                const void *q, const void *k, const void *v,
+                                const void *dout, const float *lse,
+                                const float *rpb, const int32_t *t_valid,
+                                int64_t N, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
+                                float scale, int dtype,
+                                const int64_t *qkv_strides, const int64_t *out_strides,
+                                void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Bytes of workspace na1d_fused_backward can use for these arguments (0 if it has
  * no use for one, negative status on invalid arguments). */
 int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,

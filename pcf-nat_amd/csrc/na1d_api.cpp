@@ -39,6 +39,18 @@ int check(const void *o, const void *a, const void *b, int64_t B, int64_t T, int
     return NA1D_OK;
 }
 
+// {sample, head, row} element strides of a strided entry point: multiples of 8 elements (16 bytes), rows at
+// least C apart, nothing negative.
+int check_layout(const int64_t *strides, const Geom &g, na1d::Layout &l) {
+    if (!strides) return NA1D_ERR_NULL;
+    l = na1d::Layout{strides[0], strides[1], strides[2]};
+    if (l.sample < 0 || l.head < 0 || l.row < g.C) return NA1D_ERR_SHAPE;
+    if (l.sample % 8 || l.head % 8 || l.row % 8) return NA1D_ERR_ALIGN;
+    if (l.sample > INT64_MAX / 4 / (g.B / g.H) || l.head > INT64_MAX / 4 / g.H || l.row > INT64_MAX / 4 / g.T)
+        return NA1D_ERR_SHAPE;
+    return NA1D_OK;
+}
+
 #define NA1D_CHECK(...)                     \
     Geom g;                                 \
     {                                       \
@@ -129,9 +141,10 @@ int na1d_fused_forward(void *out, float *lse, const void *q, const void *k, cons
     NA1D_CHECK(out, q, k, B, T, C, W, left, H, dtype, g);
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
-    const int st = mfma_allowed()
-                       ? na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream)
-                       : NA1D_ERR_UNSUPPORTED;
+    const na1d::Layout packed = na1d::packed_layout(g);
+    const int st = mfma_allowed() ? na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, packed, packed, scale,
+                                                          dtype, (hipStream_t)stream)
+                                  : NA1D_ERR_UNSUPPORTED;
     if (st != NA1D_ERR_UNSUPPORTED) return st;
     return na1d::generic::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream);
 }
@@ -146,13 +159,48 @@ int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb, const void *q
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
         return NA1D_ERR_ALIGN;
     if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
+    const na1d::Layout packed = na1d::packed_layout(g);
     const int st = mfma_allowed() ? na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g,
-                                                          scale, dtype, (float *)workspace,
+                                                          packed, packed, scale, dtype, (float *)workspace,
                                                           workspace ? workspace_bytes : 0, (hipStream_t)stream)
                                   : NA1D_ERR_UNSUPPORTED;
     if (st != NA1D_ERR_UNSUPPORTED) return st;
     return na1d::generic::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, scale, dtype,
                                     (hipStream_t)stream);   // the generic kernel has no use for the workspace
+}
+
+int na1d_fused_forward_strided(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+                               const int32_t *t_valid, int64_t N, int64_t H, int64_t T, int64_t C, int64_t W,
+                               int64_t left, float scale, int dtype, const int64_t *qkv_strides,
+                               const int64_t *out_strides, void *stream) {
+    if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
+    NA1D_CHECK(out, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (!v) return NA1D_ERR_NULL;
+    if (misaligned(v)) return NA1D_ERR_ALIGN;
+    na1d::Layout in, outl;
+    const int ls = check_layout(qkv_strides, g, in), lo = check_layout(out_strides, g, outl);
+    if (ls != NA1D_OK || lo != NA1D_OK) return ls != NA1D_OK ? ls : lo;
+    if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;
+    return na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, dtype, (hipStream_t)stream);
+}
+
+int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k,
+                                const void *v, const void *dout, const float *lse, const float *rpb,
+                                const int32_t *t_valid, int64_t N, int64_t H, int64_t T, int64_t C, int64_t W,
+                                int64_t left, float scale, int dtype, const int64_t *qkv_strides,
+                                const int64_t *out_strides, void *workspace, int64_t workspace_bytes,
+                                void *stream) {
+    if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
+    NA1D_CHECK(dq, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (!dk || !dv || !v || !dout || !lse) return NA1D_ERR_NULL;
+    if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(dout)) return NA1D_ERR_ALIGN;
+    if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
+    na1d::Layout in, outl;
+    const int ls = check_layout(qkv_strides, g, in), lo = check_layout(out_strides, g, outl);
+    if (ls != NA1D_OK || lo != NA1D_OK) return ls != NA1D_OK ? ls : lo;
+    if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;
+    return na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, nullptr, dout, lse, rpb, t_valid, g, in, outl, scale, dtype,
+                                 (float *)workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
 }
 
 int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,

@@ -72,6 +72,14 @@ struct Geom {
     int H;            // heads (B % H == 0); 1 for the un-fused entry points
 };
 
+// Element strides of a [samples, heads, T, C] view of a tensor whose channels are contiguous.  The packed
+// [B = samples * heads, T, C] tensor of the reference is {H*T*C, T*C, C}; a head-interleaved projection
+// output [N, T, 3, H, C] is {T*3*H*C, C, 3*H*C} behind a base pointer that selects q, k or v.
+struct Layout {
+    int64_t sample, head, row;
+};
+inline Layout packed_layout(const Geom &g) { return Layout{(int64_t)g.H * g.T * g.C, g.T * g.C, g.C}; }
+
 // Host-side launch status check.
 inline int launch_status() { return hipGetLastError() == hipSuccess ? NA1D_OK : NA1D_ERR_LAUNCH; }
 
@@ -94,12 +102,14 @@ namespace mfma {
 int qk(float *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s);
 int av(void *out, const float *attn, const void *v, const Geom &g, int dtype, hipStream_t s);
 int gather(void *out, const float *attn, const void *x, const Geom &g, int dtype, hipStream_t s);
+// `in` lays out q, k, v (and dq, dk, dv); `out` lays out out and dout.
 int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
-              const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s);
+              const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &out_layout, float scale,
+              int dtype, hipStream_t s);
 int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
               const void *out, const void *dout, const float *lse, const float *rpb,
-              const int32_t *t_valid, const Geom &g, float scale, int dtype, float *workspace,
-              int64_t workspace_bytes, hipStream_t s);
+              const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &out_layout, float scale,
+              int dtype, float *workspace, int64_t workspace_bytes, hipStream_t s);
 int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype);   // 0 when the shape is not covered
 }  // namespace mfma
 

@@ -13,11 +13,12 @@ __global__ void __launch_bounds__(kThreads)
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
-                 int strips, float scale, uint32_t strips_magic, uint32_t heads_magic) {
+                 int strips, float scale, uint32_t strips_magic, uint32_t heads_magic, Strides in, Strides outl) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = Strip<C>::kMaxTiles;
-    fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic);
+    fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
+                   in.sample, in.head, in.pitch, outl.sample, outl.head, outl.pitch);
     // dynamic LDS (fwd_lds_bytes): K and V regions of nt+2 tiles, Q region of nt tiles, 32 bias floats
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = region_bytes<C>(nt + 2);
@@ -28,29 +29,26 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t item = xcd_item(blockIdx.x, items);
-    const uint32_t b = div_by(item, strips, strips_magic);
-    const int strip = (int)(item - b * strips);
-    const uint32_t sample = div_by(b, H, heads_magic), head = b - sample * H;
-    const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
+    const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
+    const uint32_t b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
+    const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
     const int shift = NBV == 3 ? 16 : L;
 
     // resources end with the strip (plus its halo), so the fixed-size copy below
     // fetches nothing beyond what this strip needs
-    const int64_t seq_off = (int64_t)b * T * (2 * C);
-    const int seq_bytes = T * 2 * C;
-    const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
-    const Rsrc qs = make_rsrc(q + seq_off, qry_bytes), ks = make_rsrc(k + seq_off, key_bytes);
-    const Rsrc vs = make_rsrc(v + seq_off, key_bytes), os = make_rsrc(out + seq_off, seq_bytes);
+    const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
+    const int key_bytes = min(T, 16 * (i1 + 1)) * in.pitch, qry_bytes = min(T, 16 * i1) * in.pitch;
+    const Rsrc qs = make_rsrc(q + in_off, qry_bytes), ks = make_rsrc(k + in_off, key_bytes);
+    const Rsrc vs = make_rsrc(v + in_off, key_bytes), os = make_rsrc(out + out_off, T * outl.pitch);
     const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
 
     // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
     {
-        const int lane_off = direct_lane_offset<C>(wave, lane);
-        stage_direct<C, MT + 2>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off);
-        stage_direct<C, MT>(qs, 16 * i0, q_lds, nt, wave, lane_off);
-        stage_direct<C, MT + 2>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off);
+        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch);
+        stage_direct<C, MT + 2>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+        stage_direct<C, MT>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+        stage_direct<C, MT + 2>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
     }
 
@@ -145,7 +143,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
             u32x2 w;
             w.x = Mma<DT>::pack(o[ct][0] * inv, o[ct][1] * inv);
             w.y = Mma<DT>::pack(o[ct][2] * inv, o[ct][3] * inv);
-            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * (2 * C) + ct * 32 + g * 8, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * outl.pitch + ct * 32 + g * 8, 0, 0);
         }
         if (g == 0)
             __builtin_amdgcn_raw_buffer_store_b32(
@@ -155,22 +153,24 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
 
 template <class DT, int C>
 int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
-               const int32_t *t_valid, const Geom &g, float scale, hipStream_t s) {
+               const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &outl, float scale, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips) || !div_magic_ok(g.B, g.H)) return NA1D_ERR_UNSUPPORTED;
+    if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
     auto kern = window_blocks(g) == 2 ? fused_fwd_kernel<DT, C, 2> : fused_fwd_kernel<DT, C, 3>;
     const size_t lds = (size_t)2 * region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt) + 32 * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                                                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
-                                                 sp.nt, sp.strips, scale, div_magic(sp.strips), div_magic(g.H));
+                                                 sp.nt, sp.strips, scale, div_magic(sp.strips), div_magic(g.H),
+                                                 byte_strides(in), byte_strides(outl));
     return launch_status();
 }
 
 int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
-              const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s) {
+              const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &outl, float scale, int dtype,
+              hipStream_t s) {
     if (!window_blocks(g)) return NA1D_ERR_UNSUPPORTED;
-    NA1D_MFMA_DISPATCH(launch_fwd, out, lse, q, k, v, rpb, t_valid, g, scale, s);
+    NA1D_MFMA_DISPATCH(launch_fwd, out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, s);
 }
 
 // =============================================================================
@@ -226,12 +226,13 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes, uint32_t strips_magic,
-                 uint32_t heads_magic) {
+                 uint32_t heads_magic, Strides in, Strides outl) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
-                   drpb_partial, kv_bytes, strips_magic, heads_magic);
+                   drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, outl.sample,
+                   outl.head, outl.pitch);
     constexpr int kRowsQ = (MT + 2) * 16;
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
@@ -254,28 +255,27 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t item = xcd_item(blockIdx.x, items);
-    const uint32_t b = div_by(item, strips, strips_magic);
-    const int strip = (int)(item - b * strips);
-    const uint32_t sample = div_by(b, H, heads_magic), head = b - sample * H;
-    const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
+    const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
+    const uint32_t item = wi.item, b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
+    const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
     const int shift = NBV == 3 ? 16 : L;
 
-    const int64_t seq_off = (int64_t)b * T * (2 * C);
-    const int seq_bytes = T * 2 * C;
+    const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
     {
-        const int key_bytes = min(T, 16 * (i1 + 2)) * 2 * C, qry_bytes = min(T, 16 * (i1 + 1)) * 2 * C;
-        const Rsrc ks = make_rsrc(k + seq_off, key_bytes), vs = make_rsrc(v + seq_off, key_bytes);
-        const Rsrc qs = make_rsrc(q + seq_off, qry_bytes), gs = make_rsrc(dout + seq_off, qry_bytes);
+        const int key_bytes = min(T, 16 * (i1 + 2)) * in.pitch;
+        const int qry_rows = min(T, 16 * (i1 + 1));
+        const Rsrc ks = make_rsrc(k + in_off, key_bytes), vs = make_rsrc(v + in_off, key_bytes);
+        const Rsrc qs = make_rsrc(q + in_off, qry_rows * in.pitch), gs = make_rsrc(dout + out_off, qry_rows * outl.pitch);
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
-        const int lane_off = direct_lane_offset<C>(wave, lane);
+        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch);
+        const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch);
         // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * i0 - 16 + tid) * 4, 0, 0, 0);
-        stage_direct<C, MT + 4>(ks, 16 * i0 - 32, k_lds, nt + 4, wave, lane_off);
-        stage_direct<C, MT + 2>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off);
-        stage_direct<C, MT + 4>(vs, 16 * i0 - 32, v_lds, nt + 4, wave, lane_off);
-        stage_direct<C, MT + 2>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off);
+        stage_direct<C, MT + 4>(ks, 16 * i0 - 32, k_lds, nt + 4, wave, lane_off, in.pitch);
+        stage_direct<C, MT + 2>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
+        stage_direct<C, MT + 4>(vs, 16 * i0 - 32, v_lds, nt + 4, wave, lane_off, in.pitch);
+        stage_direct<C, MT + 2>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
     }
 
@@ -298,7 +298,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 
     // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
-    const Rsrc dqs = make_rsrc(dq + seq_off, seq_bytes);
+    const Rsrc dqs = make_rsrc(dq + in_off, T * in.pitch);
     u32x2 sc[TPW][2][2];                // [tile of this wave][X/Y slot set][P / dS], rounded to 16 bit
 #pragma unroll
     for (int jt = 0; jt < TPW; ++jt) {
@@ -389,7 +389,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             u32x2 w;
             w.x = Mma<DT>::pack(acc[ct][0] * scale, acc[ct][1] * scale);
             w.y = Mma<DT>::pack(acc[ct][2] * scale, acc[ct][3] * scale);
-            __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * (2 * C) + ct * 32 + g * 8, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * in.pitch + ct * 32 + g * 8, 0, 0);
         }
     }
 
@@ -448,8 +448,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     }
     const int sc_lane = (4 * g + (n >> 2)) * 32 + (n & 3) * 8;       // transposed read of a score tile
     const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
-    const Rsrc dks = make_rsrc(dk + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
-    const Rsrc dvs = make_rsrc(dv + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
+    const Rsrc dks = make_rsrc(dk + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
+    const Rsrc dvs = make_rsrc(dv + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
     const int kp_lo = i0 + (shift == 16 ? 1 : 0), kp_hi = i1 - (shift == 0 ? 1 : 0);
     for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
         f32x4 acck[CT], accv[CT];
@@ -476,7 +476,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                 acck[ct] = Mma<DT>::k16(read_tr(qtile + qry_tr.off[ct]), db, acck[ct]);
             }
         }
-        const int row_off = (16 * (kp - i0) - shift + n) * (2 * C);     // outside the strip -> dropped
+        const int row_off = (16 * (kp - i0) - shift + n) * in.pitch;    // outside the strip -> dropped
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             u32x2 wk, wv;
@@ -503,9 +503,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 template <class DT, int C>
 int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
                const void *dout, const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g,
-               float scale, float *workspace, int64_t workspace_bytes, hipStream_t s) {
+               const Layout &in, const Layout &outl, float scale, float *workspace, int64_t workspace_bytes,
+               hipStream_t s) {
     const Split sp = make_split(g.B, g.T, StripBwd<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips) || !div_magic_ok(g.B, g.H)) return NA1D_ERR_UNSUPPORTED;
+    if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
     float *partial = nullptr;
     if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
     auto kern = window_blocks(g) == 2 ? fused_bwd_kernel<DT, C, 2> : fused_bwd_kernel<DT, C, 3>;
@@ -518,7 +519,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                                                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
                                                  t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
                                                  sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
-                                                 div_magic(g.H));
+                                                 div_magic(g.H), byte_strides(in), byte_strides(outl));
     if (partial && drpb)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();
@@ -531,10 +532,11 @@ int64_t bwd_workspace(const Geom &g) {
 
 int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
               const void *out, const void *dout, const float *lse, const float *rpb, const int32_t *t_valid,
-              const Geom &g, float scale, int dtype, float *workspace, int64_t workspace_bytes, hipStream_t s) {
+              const Geom &g, const Layout &in, const Layout &outl, float scale, int dtype, float *workspace,
+              int64_t workspace_bytes, hipStream_t s) {
     (void)out;   // delta is recomputed from P and dP; O is not needed
     if (!window_blocks(g)) return NA1D_ERR_UNSUPPORTED;
-    NA1D_MFMA_DISPATCH(launch_bwd, dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, scale, workspace,
+    NA1D_MFMA_DISPATCH(launch_bwd, dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, workspace,
                        workspace_bytes, s);
 }
 

@@ -139,21 +139,25 @@ static_assert(kWaves % 4 == 0, "chunk -> swizzle phase mapping assumes a multipl
 template <int C> constexpr int region_bytes(int ntiles) {
     return (ntiles * Lds<C>::kTileBytes + kChunk - 1) / kChunk * kChunk;
 }
-template <int C> __device__ inline int direct_lane_offset(int wave, int lane) {
+// `pitch` is the distance in bytes between consecutive rows in memory (2*C when the
+// rows are packed).
+template <int C> __device__ inline int direct_lane_offset(int wave, int lane, int pitch = Lds<C>::kRowBytes) {
     const int u = wave * 64 + lane;      // 16-byte unit inside chunks wave, wave + 4, ...
     const int su = u % Lds<C>::kUnits;
-    return (lane - su + (su ^ Lds<C>::swz(u / Lds<C>::kUnits))) * 16;
+    return (lane / Lds<C>::kUnits) * pitch + (su ^ Lds<C>::swz(u / Lds<C>::kUnits)) * 16;
 }
 template <int C, int NTILES>
-__device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, int ntiles, int wave, int lane_off) {
+__device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, int ntiles, int wave, int lane_off,
+                                    int pitch = Lds<C>::kRowBytes) {
     constexpr int kRounds = (region_bytes<C>(NTILES) / kChunk + kWaves - 1) / kWaves;
+    constexpr int kChunkRows = kChunk / Lds<C>::kRowBytes;
     const int chunks = region_bytes<C>(ntiles) / kChunk;
-    const int base = row_lo * Lds<C>::kRowBytes + lane_off;
+    const int base = row_lo * pitch + lane_off, step = kChunkRows * pitch;
 #pragma unroll
     for (int j = 0; j < kRounds; ++j) {
         const int c = j * kWaves + wave;
         if (c < chunks)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * kChunk), 16, base + c * kChunk, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * kChunk), 16, base + c * step, 0, 0, 0);
     }
 }
 __device__ inline void wait_direct() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
@@ -314,6 +318,39 @@ inline Split make_split(int64_t B, int64_t T, int max_tiles) {
     s.strips = (s.tiles + s.nt - 1) / s.nt;
     s.items = B * s.strips;
     return s;
+}
+
+// Byte strides of one tensor family as the kernels take them.
+struct Strides {
+    int64_t sample, head;   // from one sample / head to the next
+    int pitch;              // from one row to the next
+};
+inline Strides byte_strides(const Layout &l) { return Strides{2 * l.sample, 2 * l.head, (int)(2 * l.row)}; }
+// Offsets inside one sequence are 32-bit: the rows of a sequence, plus the halo rows the copies ask for
+// beyond its end, must span less than 2^30 bytes.
+inline bool strides_ok(const Layout &l, const Geom &g) { return l.row >= g.C && g.T + 96 <= (1 << 29) / l.row; }
+inline bool items_ok(const Split &sp, const Geom &g) {
+    return sp.items <= 0x7fffff00LL && div_magic_ok(sp.items, g.H) && div_magic_ok(sp.items, sp.strips);
+}
+
+// Workgroup id -> (sample, head, strip).  Heads vary fastest, then strips: workgroups that run side by side
+// touch the same rows of a head-interleaved tensor (and neighbouring strips, which share halo rows), and
+// xcd_item() keeps such a run of ids on one XCD, i.e. behind one L2.
+struct WorkItem {
+    uint32_t sample, head, item;   // item = (sample * H + head) * strips + strip: the d rpb partial-sum row
+    int strip;
+};
+__device__ inline uint32_t xcd_item(uint32_t wg, uint32_t items);
+__device__ inline WorkItem work_item(uint32_t wg, uint32_t items, int strips, uint32_t strips_magic, int H,
+                                     uint32_t heads_magic) {
+    const uint32_t lin = xcd_item(wg, items);
+    const uint32_t rest = div_by(lin, H, heads_magic);
+    WorkItem w;
+    w.head = lin - rest * H;
+    w.sample = div_by(rest, strips, strips_magic);
+    w.strip = (int)(rest - w.sample * strips);
+    w.item = (w.sample * H + w.head) * strips + w.strip;
+    return w;
 }
 
 // Workgroup id -> work item, so that consecutive items (neighbouring strips of a

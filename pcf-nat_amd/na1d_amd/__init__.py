@@ -5,4 +5,4 @@
 ``_lib``   - ctypes binding of the C-ABI library ``libna1d.so``
 """
 from .nattn import getNA1dFunction  # noqa: F401
-from .fused import na1d_fused  # noqa: F401
+from .fused import na1d_fused, na1d_fused_qkv  # noqa: F401

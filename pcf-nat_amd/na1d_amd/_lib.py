@@ -21,7 +21,9 @@ _i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_
 _UNFUSED = ("na1d_qk_forward", "na1d_av_forward", "na1d_q_backward", "na1d_k_backward",
             "na1d_a_backward", "na1d_v_backward")
 SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_backward_workspace_bytes",
+                      "na1d_fused_forward_strided", "na1d_fused_backward_strided",
                       "na1d_version", "na1d_status_string")
+UNSUPPORTED = -8
 
 _lib = None
 
@@ -52,6 +54,10 @@ def load():
                                        _i64, _i64, _i64, _i64, _i64, _i64, _f32, _int, _ptr]
     lib.na1d_fused_backward.restype = _int
     lib.na1d_fused_backward.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _ptr, _i64, _ptr]
+    lib.na1d_fused_forward_strided.restype = _int
+    lib.na1d_fused_forward_strided.argtypes = [_ptr] * 7 + [_i64] * 6 + [_f32, _int, _ptr, _ptr, _ptr]
+    lib.na1d_fused_backward_strided.restype = _int
+    lib.na1d_fused_backward_strided.argtypes = [_ptr] * 11 + [_i64] * 6 + [_f32, _int, _ptr, _ptr, _ptr, _i64, _ptr]
     lib.na1d_fused_backward_workspace_bytes.restype = _i64
     lib.na1d_fused_backward_workspace_bytes.argtypes = [_i64] * 6 + [_int]
     lib.na1d_version.restype = _int
@@ -118,3 +124,37 @@ def call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid,
                                      _p(lse), _p(rpb), _p(t_valid), B, H, T, C, W, left, scale,
                                      dtype_tag(q.dtype), _p(workspace), ws_bytes, _stream(dq))
     check(st, "na1d_fused_backward")
+
+
+def _strides3(view):
+    """{sample, head, row} element strides of a ``[N, H, T, C]`` view with contiguous channels."""
+    assert view.dim() == 4 and (view.shape[3] == 1 or view.stride(3) == 1), "channels must be contiguous"
+    return (_i64 * 3)(view.stride(0), view.stride(1), view.stride(2))
+
+
+def call_fused_forward_strided(out, lse, q, k, v, rpb, t_valid, W, left, scale):
+    """q, k, v, out: ``[N, H, T, C]`` views (q, k, v with equal strides).  Returns the status so that the
+    caller can pack the tensors when no strided kernel covers the shape (``UNSUPPORTED``)."""
+    lib = load()
+    N, H, T, C = q.shape
+    assert q.stride() == k.stride() == v.stride()
+    with torch.cuda.device(out.device):
+        st = lib.na1d_fused_forward_strided(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid), N, H, T, C, W,
+                                            left, scale, dtype_tag(q.dtype), _strides3(q), _strides3(out), _stream(out))
+    if st != UNSUPPORTED:
+        check(st, "na1d_fused_forward_strided")
+    return st
+
+
+def call_fused_backward_strided(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, W, left, scale, workspace=None):
+    lib = load()
+    N, H, T, C = q.shape
+    assert q.stride() == k.stride() == v.stride() == dq.stride() == dk.stride() == dv.stride()
+    ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
+    with torch.cuda.device(dq.device):
+        st = lib.na1d_fused_backward_strided(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(dout), _p(lse),
+                                             _p(rpb), _p(t_valid), N, H, T, C, W, left, scale, dtype_tag(q.dtype),
+                                             _strides3(q), _strides3(dout), _p(workspace), ws_bytes, _stream(dq))
+    if st != UNSUPPORTED:
+        check(st, "na1d_fused_backward_strided")
+    return st

@@ -86,6 +86,28 @@ def test_fused_entry_points_validate():
     assert w(4, 3, 8, 16, 5, 2, 0) == -5 and w(4, 2, 8, 16, 99, 2, 0) == -4
 
 
+def test_strided_entry_points_validate():
+    lib = _lib.load()
+    P, ok = ctypes.c_void_p, ctypes.c_void_p(0x1000)
+    S = lambda *v: (ctypes.c_int64 * 3)(*v)
+    qkv, out = S(8 * 3 * 2 * 16, 16, 3 * 2 * 16), S(8 * 2 * 16, 16, 2 * 16)     # [N, T, 3, H, C] / [N, T, H*C], T=8, H=2, C=16
+    f = lib.na1d_fused_forward_strided
+    args = lambda **kw: [kw.get("o", ok), None, ok, ok, kw.get("v", ok), None, None, kw.get("N", 2), 2, 8, kw.get("C", 16),
+                         kw.get("W", 5), 2, 1.0, 0, kw.get("qs", qkv), kw.get("os", out), None]
+    assert f(*args(qs=None)) == -1 and f(*args(os=None)) == -1 and f(*args(v=None)) == -1
+    assert f(*args(qs=S(768, 16, 8))) == -5          # rows closer than C
+    assert f(*args(qs=S(768, 12, 96))) == -6         # head stride not a multiple of 8 elements
+    assert f(*args(os=S(-256, 16, 32))) == -5
+    assert f(*args(C=20)) == -3 and f(*args(W=99)) == -4 and f(*args(N=-1)) == -5
+    assert f(*args(N=0)) == 0                        # nothing to do
+    assert f(*args(C=24, qs=S(8 * 3 * 2 * 24, 24, 3 * 2 * 24), os=S(8 * 2 * 24, 24, 48))) == -8   # no strided kernel for C=24
+    b = lib.na1d_fused_backward_strided
+    bargs = lambda **kw: [ok, ok, ok, None, ok, ok, ok, kw.get("g", ok), kw.get("lse", ok), None, None, 2, 2, 8, 16, 5, 2,
+                          1.0, 0, kw.get("qs", qkv), out, kw.get("ws", None), 64, None]
+    assert b(*bargs(lse=None)) == -1 and b(*bargs(g=None)) == -1 and b(*bargs(qs=None)) == -1
+    assert b(*bargs(ws=P(0x1008))) == -6
+
+
 def test_python_layer_mirrors_reference_entry_points():
     """Names, dispatch and asserts of na1d_tensorcore/nattn.py:128-137."""
     qk, av = nattn.getNA1dFunction(C=16, dilation=1, dtype=torch.bfloat16)

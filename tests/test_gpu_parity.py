@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from oracle import na1d_oracle as O
-from na1d_amd import _lib, nattn, na1d_fused
+from na1d_amd import _lib, nattn, na1d_fused, na1d_fused_qkv
 from na1d_amd.fused import na1d_fused_forward_lse
 from _util import TOL, dev, make_inputs, seeded_scores
 
@@ -166,6 +166,70 @@ def test_fused_forward_backward_matches_oracle(geom, dtype):
     assert _err(rd.grad, wr) < tol, "drpb"
     _, lse = na1d_fused_forward_lse(qd.detach(), kd.detach(), vd.detach(), W, L, rd.detach(), t_valid.cuda(), H)
     assert torch.allclose(lse.cpu(), want_lse, atol=2e-3, rtol=1e-4), "LSE"
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", [g for g in FUSED_GEOMS if g[2] > 1], ids=lambda g: "x".join(map(str, g)))
+def test_fused_on_projection_layout_matches_oracle_and_packed_operator(geom, dtype):
+    """q, k, v read in place from a [N, T, 3, H, C] projection output, out written as [N, T, H*C]: against
+    the oracle on the packed copies, and bit for bit against the packed operator where the same kernels serve
+    both (shapes they do not cover go through the packing fallback)."""
+    N, H, T, C, W, L = geom
+    g = torch.Generator().manual_seed(12)
+    qkv = (torch.randn(N, T, 3, H, C, generator=g) * (C ** -0.25)).to(dtype)
+    do = torch.randn(N, T, H * C, generator=g).to(dtype)
+    rpb = torch.randn(H, W, generator=g) * 0.5
+    pad = torch.tensor([0, T // 2, T][:N] + [1] * max(0, N - 3))
+    t_valid = (T - pad).to(torch.int32).cuda()
+
+    xd = qkv.cuda().requires_grad_(True)
+    rd = rpb.cuda().requires_grad_(True)
+    out = na1d_fused_qkv(xd, W, L, rpb=rd, t_valid=t_valid)
+    assert out.shape == (N, T, H * C) and out.is_contiguous()
+    out.backward(do.cuda())
+
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3).contiguous().view(N * H, T, C) for i in range(3))   # the reference's packing
+    dop = do.view(N, T, H, C).permute(0, 2, 1, 3).contiguous().view(N * H, T, C)
+    unpack = lambda z: z.reshape(N, H, T, C).permute(0, 2, 1, 3)
+    want_o, _, _ = O.na1d_forward(q.float(), k.float(), v.float(), W, L, rpb, pad, H)
+    wq, wk, wv, wr = O.na1d_backward(q.float(), k.float(), v.float(), dop.float(), W, L, rpb, pad, H)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float().view(N, T, H, C), unpack(want_o)) < tol, "O"
+    for i, (name, want) in enumerate((("dQ", wq), ("dK", wk), ("dV", wv))):
+        assert O.rel_l2(xd.grad[:, :, i].float(), unpack(want)) < tol, name
+    assert _err(rd.grad, wr) < tol, "drpb"
+
+    qd, kd, vd = (z.cuda().requires_grad_(True) for z in (q, k, v))
+    packed = na1d_fused(qd, kd, vd, W, L, rpb=rpb.cuda(), t_valid=t_valid, num_heads=H)
+    packed.backward(dop.cuda())
+    assert torch.equal(out.view(N, T, H, C), unpack(packed))
+    for i, z in enumerate((qd, kd, vd)):
+        assert torch.equal(xd.grad[:, :, i], unpack(z.grad))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_strided_entry_points_leave_the_gaps_alone(dtype):
+    """Rows 3*H*C apart with the k and v slots (and a pad column) between them: nothing but the addressed
+    rows may be written."""
+    N, H, T, C, W, L = 2, 3, 50, 16, 27, 13
+    g = torch.Generator().manual_seed(5)
+    buf = torch.randn(N, T, 3, H, C + 8, generator=g).to(dtype).cuda()        # 8 pad channels per head row
+    views = [buf[:, :, i, :, :C].permute(0, 2, 1, 3) for i in range(3)]       # [N, H, T, C], row stride 3*H*(C+8)
+    obuf = torch.full((N, T, H, C + 8), 7.0, dtype=dtype, device="cuda")
+    out = obuf[..., :C].permute(0, 2, 1, 3)
+    lse = torch.empty(N * H, T, device="cuda")
+    assert _lib.call_fused_forward_strided(out, lse, *views, None, None, W, L, 1.0) == 0
+    assert torch.all(obuf[..., C:] == 7.0)
+    packed = [z.contiguous().view(N * H, T, C) for z in views]
+    want, _ = na1d_fused_forward_lse(*packed, W, L)
+    assert torch.equal(out.contiguous().view(N * H, T, C), want)
+
+    gbuf = torch.full_like(buf, float("nan"))
+    gviews = [gbuf[:, :, i, :, :C].permute(0, 2, 1, 3) for i in range(3)]
+    do = torch.randn(N, H, T, C, generator=g).to(dtype).cuda()
+    assert _lib.call_fused_backward_strided(*gviews, None, *views, do, lse, None, None, W, L, 1.0) == 0
+    assert torch.isnan(gbuf[..., C:]).all()
+    assert not torch.isnan(gbuf[..., :C]).any()
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
