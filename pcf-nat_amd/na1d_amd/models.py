@@ -8,6 +8,8 @@ models/Pooling.py, models/SoftMaxLoss.py:99-138) in plain torch.nn, built so tha
   checkpoint loads with ``load_state_dict``);
 * the neighbourhood attention runs through this package's operator:
   ``na="fused"`` (one HIP kernel each way, no mask or score tensor),
+  ``na="fused_qkv"`` (the same kernels reading q, k, v in place from a token-major qkv projection and
+  writing the merged heads directly: no head split / merge copies, no ``q * scale`` pass),
   ``na="unfused"`` (the reference's own chain QK -> +rpb -> +mask -> softmax -> AV
   through the drop-in Functions), or any callable with the signature of
   :func:`na1d_amd.na1d_fused` (tests pass a CPU function here to build a twin).
@@ -26,7 +28,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .fused import na1d_fused
+from .fused import na1d_fused, na1d_fused_qkv
 from .nattn import getNA1dFunction
 
 MASK_VALUE = -100.0   # PCF_NATransformer.py:98
@@ -163,6 +165,24 @@ def _merge_heads(x, n, num_heads, channels_first):
     return x.transpose(1, 2).contiguous().view(n, t, num_heads * hd)
 
 
+def _dense_weight(proj):
+    """[out, in] matrix of a per-token projection: a Linear's weight, or a grouped 1x1 convolution's blocks on
+    the diagonal."""
+    if isinstance(proj, nn.Linear):
+        return proj.weight
+    w = proj.weight[:, :, 0]
+    return w if proj.groups == 1 else torch.block_diag(*w.view(proj.groups, w.shape[0] // proj.groups, w.shape[1]))
+
+
+def _qkv_channel_order(dim, groups, device):
+    """Output channel of the channels-first qkv convolution that holds (which, head-major channel f): the inverse
+    of the view/transpose chain of :func:`_split_heads` (PCF_NATransformer.py:126-129), as a row index."""
+    f = torch.arange(dim, device=device)
+    per = dim // groups
+    oc = ((f % per) * groups + f // per) * 3                      # which = 0
+    return torch.cat([oc, oc + 1, oc + 2])
+
+
 def _window_mask(T, W, left, padding, dtype, device):
     """[N, T, W] additive mask of PCF_NATransformer.py:87-99."""
     if padding is None:
@@ -203,9 +223,11 @@ class NAttention(nn.Module):
         n = x.shape[0]
         t = x.shape[-1] if self.channels_first else x.shape[1]
         h, w, left = self.num_heads, self.win_size, self.left
+        t_valid = None if padding is None else (t - padding).to(torch.int32)
+        if self.na == "fused_qkv":
+            return self._forward_token_major(x, n, t, t_valid)
         q, k, v = _split_heads(self.qkv(x), h, self.groups, self.channels_first)
         q = q * self.scale                                   # in the activation dtype, as the reference does (:141)
-        t_valid = None if padding is None else (t - padding).to(torch.int32)
         if callable(self.na):
             out = self.na(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h)
         elif self.na == "fused":
@@ -217,6 +239,24 @@ class NAttention(nn.Module):
             attn = torch.softmax(attn.view(n * h, t, w), dim=-1)
             out = self.NA1d_AV_Function.apply(attn, v, w, left, 1)
         return self.proj(_merge_heads(out, n, h, self.channels_first))
+
+    def _forward_token_major(self, x, n, t, t_valid):
+        """The same layer with the operator reading the qkv projection in place.  Tokens-first models have the
+        layout already; channels-first ones get it by running the two 1x1 convolutions as matrix products whose
+        output rows are ordered (which, head, channel) - the same parameters, the same arithmetic, no copies."""
+        h = self.num_heads
+        if self.channels_first:
+            order = _qkv_channel_order(self.dim, self.groups, x.device)
+            wq = _dense_weight(self.qkv).index_select(0, order).t().unsqueeze(0).expand(n, -1, -1)
+            qkv = torch.baddbmm(self.qkv.bias.index_select(0, order).view(1, 1, -1), x.transpose(1, 2), wq)   # [N, T, 3*dim]
+        else:
+            qkv = self.qkv(x)
+        out = na1d_fused_qkv(qkv.view(n, t, 3, h, self.dim // h), self.win_size, self.left,
+                             rpb=self.relative_position_bias, t_valid=t_valid, scale=self.scale)      # [N, T, dim]
+        if self.channels_first:
+            wp = _dense_weight(self.proj).unsqueeze(0).expand(n, -1, -1)
+            return torch.baddbmm(self.proj.bias.view(1, -1, 1), wp, out.transpose(1, 2))                      # [N, dim, T]
+        return self.proj(out)
 
 
 class GlobalAttention(nn.Module):

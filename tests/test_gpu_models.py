@@ -33,7 +33,7 @@ def _twin(factory, dtype, seed=0, **kw):
     return cpu
 
 
-@pytest.mark.parametrize("na", ["fused", "unfused"])
+@pytest.mark.parametrize("na", ["fused", "fused_qkv", "unfused"])
 def test_pcf_nat_4x4_inference_bf16(na):
     """cfg3: 80-dim fbank, 200 frames, bf16; pooled speaker embedding vs the CPU twin."""
     cpu = _twin(models.PCF_NATransformer, torch.bfloat16).eval()
@@ -51,10 +51,11 @@ def test_pcf_nat_4x4_inference_bf16(na):
     assert cos.min().item() >= 0.999, cos
 
 
-def test_pcf_nat_6x4_variable_length_bf16():
+@pytest.mark.parametrize("na", ["fused", "fused_qkv"])
+def test_pcf_nat_6x4_variable_length_bf16(na):
     """cfg4: lengths uniform in 300..2000 frames, padded to the longest, masks from `lens`."""
     cpu = _twin(models.pcf_nat_6x4, torch.bfloat16).eval()
-    gpu = models.pcf_nat_6x4(na="fused", dtype=torch.bfloat16)
+    gpu = models.pcf_nat_6x4(na=na, dtype=torch.bfloat16)
     gpu.load_state_dict(cpu.state_dict())
     gpu = gpu.cuda().eval()
     g = torch.Generator().manual_seed(2)
@@ -72,11 +73,12 @@ def test_pcf_nat_6x4_variable_length_bf16():
     assert cos.min().item() >= 0.999, cos
 
 
-def test_mfa_nat_4x4_training_step_fp16():
+@pytest.mark.parametrize("na", ["fused", "fused_qkv"])
+def test_mfa_nat_4x4_training_step_fp16(na):
     """cfg5: forward+backward through NA1D under fp16 autocast with a GradScaler, AAM sub-centre head over
     5994 classes, one SGD-Nesterov step; loss and parameter gradients vs the CPU fp32 twin."""
     cpu = _twin(models.MFA_NATransformer, torch.float16, frames=200).train()
-    gpu = models.MFA_NATransformer(na="fused", dtype=torch.float16, frames=200)
+    gpu = models.MFA_NATransformer(na=na, dtype=torch.float16, frames=200)
     gpu.load_state_dict(cpu.state_dict())
     gpu = gpu.cuda().train()
     torch.manual_seed(3)

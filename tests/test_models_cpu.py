@@ -69,3 +69,23 @@ def test_first_step_loss_matches_published_log():
     head = models.ArcMarginSubCenters(192, 17982, m=0.2, s=32.0, subcenters=3)
     loss, _ = head(torch.randn(256, 192), torch.randint(0, 17982, (256,)))
     assert 16.0 < loss.item() < 20.0
+
+
+@pytest.mark.parametrize("groups", [1, 2, 4, 8])
+def test_token_major_projections_equal_the_grouped_convolutions(groups):
+    """The fused_qkv path runs the channels-first 1x1 convolutions as matrix products with reordered rows; the
+    result must be the reference's head split (PCF_NATransformer.py:126-139) / the plain output projection."""
+    torch.manual_seed(groups)
+    n, dim, t, heads = 2, 64, 11, 4
+    layer = models.NAttention(t, dim, heads, 7, groups=groups, channels_first=True, na="fused_qkv")
+    x = torch.randn(n, dim, t)
+    want = models._split_heads(layer.qkv(x), heads, groups, True)                       # [3, N*H, T, hd]
+    order = models._qkv_channel_order(dim, groups, x.device)
+    wq = models._dense_weight(layer.qkv).index_select(0, order).t().unsqueeze(0).expand(n, -1, -1)
+    qkv = torch.baddbmm(layer.qkv.bias.index_select(0, order).view(1, 1, -1), x.transpose(1, 2), wq)
+    got = qkv.view(n, t, 3, heads, dim // heads).permute(2, 0, 3, 1, 4).reshape(3, n * heads, t, dim // heads)
+    assert torch.allclose(got, want, atol=1e-5)
+    o = torch.randn(n, t, dim)
+    wp = models._dense_weight(layer.proj).unsqueeze(0).expand(n, -1, -1)
+    got = torch.baddbmm(layer.proj.bias.view(1, -1, 1), wp, o.transpose(1, 2))
+    assert got.is_contiguous() and torch.allclose(got, layer.proj(o.transpose(1, 2)), atol=1e-5)
