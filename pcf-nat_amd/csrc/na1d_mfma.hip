@@ -239,8 +239,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     static_assert(kRowsQ <= kThreads, "one lane per staged lse row");
     // dynamic LDS (see launch_bwd): [K region | V region] of nt+4 tiles each (rows 16*i0 - 32 ...), reused after
     // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt+2 tiles (rows 16*i0 - 16 ...); lse
-    // of the query-side rows; 32 bias floats; and - only when d rpb is wanted - per-lane partial sums and 8
-    // partial sums per slot
+    // of the query-side rows; 32 bias floats; and - only when d rpb is wanted - 32 slot sums per wave
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = region_bytes<C>(nt + 4), qry_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
@@ -250,8 +249,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
     LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
     LDS_PTR(float) bias_lds = lse_lds + kThreads;
-    LDS_PTR(float) rpart = bias_lds + 32;          // [kWaves * 8][64]
-    LDS_PTR(float) rsum = rpart + kWaves * 8 * 64; // [8][32]
+    LDS_PTR(float) rsum = bias_lds + 32;           // [kWaves][32] d rpb slot sums per wave
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -393,14 +391,29 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
 
-    // d rpb: the window slot of each of a lane's 8 score registers is the same for every tile, so the
-    // lane keeps running sums; they are folded across lanes and waves through LDS in a fixed order.
+    // d rpb: the window slot of each of a lane's 8 score registers is the same for every tile, so the lane
+    // keeps running sums.  Register r of lane (n, g) holds key a = 4g + r of its block against query n, and the
+    // slot depends on a - n only: slot = (a - n + L - shift) mod 32 for set X, 16 more for set Y.  A lane
+    // permutation lines the 16 diagonals a - n = d (mod 16) up in lane d; the two members of a class, a - n = d
+    // and a - n = d - 16, are told apart by a >= d and go to slots 16 apart, set X and set Y crosswise.  What is
+    // left is a sum over the 16 keys a: four registers, then the four lane groups.  Fixed order throughout.
     if (drpb) {
+        float s0 = 0.f, s1 = 0.f;         // slots (n + L - shift) mod 32 and 16 further, n = this lane's class
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            rpart[(wave * 8 + r) * 64 + lane] = racc_x[r];
-            rpart[(wave * 8 + 4 + r) * 64 + lane] = racc_y[r];
+            const int a = 4 * g + r;
+            const int from = (16 * g + ((a - n) & 15)) * 4;
+            const float x = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(racc_x[r])));
+            const float y = __int_as_float(__builtin_amdgcn_ds_bpermute(from, __float_as_int(racc_y[r])));
+            const bool upper = a >= n;     // a - n = d, else d - 16
+            s0 += upper ? x : y;
+            s1 += upper ? y : x;
         }
+        s0 = xor_sum(s0);
+        s1 = xor_sum(s1);
+        const int slot = (n + L - shift) & 31;
+        if (g == 0) rsum[wave * 32 + slot] = s0;
+        if (g == 1) rsum[wave * 32 + ((slot + 16) & 31)] = s1;
     }
 
     __syncthreads();                    // every wave is done with K and V: their regions become the score tiles
@@ -414,25 +427,6 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 #pragma unroll
             for (int pd = 0; pd < 2; ++pd) *reinterpret_cast<LDS_PTR(u32x2)>(t + (xy * 2 + pd) * kScoreTile) = sc[jt][xy][pd];
     }
-    if (drpb) {
-        // thread (j, p): slot j, wave p/2, registers r = 2*(p&1), 2*(p&1)+1; the lane (n, g) whose register r
-        // holds slot j has n = 4g + r - shift + L - j (+32: merged block 2, +16: block 1)
-        const int j = tid & 31, p = tid >> 5, w = p >> 1;
-        float sum = 0.f;
-#pragma unroll
-        for (int rr = 0; rr < 2; ++rr) {
-            const int r = 2 * (p & 1) + rr;
-#pragma unroll
-            for (int gg = 0; gg < 4; ++gg) {
-                const int na = 4 * gg + r - shift + L - j;
-                const int nx = (NBV == 3 && na < 0) ? na + 32 : na, ny = na + 16;
-                if (nx >= 0 && nx < 16) sum += rpart[(w * 8 + r) * 64 + 16 * gg + nx];
-                if (ny >= 0 && ny < 16) sum += rpart[(w * 8 + 4 + r) * 64 + 16 * gg + ny];
-            }
-        }
-        rsum[p * 32 + j] = sum;
-    }
-    
     __syncthreads();
 
     // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
@@ -489,10 +483,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
 
-    if (drpb && tid < W) {              // rsum was complete at the barrier before pass 2
+    if (drpb && tid < W) {              // rsum was complete at the barriers before pass 2
         float t = 0.f;
 #pragma unroll
-        for (int p = 0; p < 8; ++p) t += rsum[p * 32 + tid];
+        for (int w = 0; w < kWaves; ++w) t += rsum[w * 32 + tid];
         if (drpb_partial)
             drpb_partial[(size_t)item * kPartialStride + tid] = t;   // folded by drpb_reduce_kernel
         else
@@ -513,7 +507,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
     const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 4), (sp.nt + 2) * 4 * 512);
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
-                       (kThreads + 32 + (drpb ? kWaves * 8 * 64 + 8 * 32 : 0)) * sizeof(float);
+                       (kThreads + 32 + (drpb ? kWaves * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                                                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
