@@ -19,7 +19,9 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     constexpr int MT = Strip<C>::kMaxTiles;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, outl.sample, outl.head, outl.pitch);
-    // dynamic LDS (fwd_lds_bytes): K and V regions of nt+2 tiles, Q region of nt tiles, 32 bias floats
+    // dynamic LDS (launch_fwd): K and V regions of nt+2 tiles starting one tile before the strip (row 16*i0 - 16:
+    // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
+    // forward is not short of LDS), Q region of nt tiles, 32 bias floats
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
@@ -237,11 +239,12 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
     static_assert(kRowsQ <= kThreads, "one lane per staged lse row");
-    // dynamic LDS (see launch_bwd): [K region | V region] of nt+4 tiles each (rows 16*i0 - 32 ...), reused after
+    // dynamic LDS (see launch_bwd): [K region | V region] of nt+1+NBV tiles each, starting at the first key of
+    // query tile i0-1 (row 16*(i0-1) - shift, so that virtual key blocks are whole tiles of the region), reused after
     // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt+2 tiles (rows 16*i0 - 16 ...); lse
     // of the query-side rows; 32 bias floats; and - only when d rpb is wanted - 32 slot sums per wave
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int key_region = region_bytes<C>(nt + 4), qry_region = region_bytes<C>(nt + 2);
+    const int key_region = region_bytes<C>(nt + 1 + NBV), qry_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
     LDS_PTR(char) sc_lds = k_lds;                  // score tiles [(tq*2 + X/Y)*2 + P/dS]
@@ -270,9 +273,9 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch);
         // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * i0 - 16 + tid) * 4, 0, 0, 0);
-        stage_direct<C, MT + 4>(ks, 16 * i0 - 32, k_lds, nt + 4, wave, lane_off, in.pitch);
+        stage_direct<C, MT + 1 + NBV>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
         stage_direct<C, MT + 2>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
-        stage_direct<C, MT + 4>(vs, 16 * i0 - 32, v_lds, nt + 4, wave, lane_off, in.pitch);
+        stage_direct<C, MT + 1 + NBV>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
         stage_direct<C, MT + 2>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
     }
@@ -284,8 +287,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 
     RowLane<C> key_lane, qry_lane;      // row operands: virtual key block rows / query tile rows
     TrLane<C> key_tr, qry_tr;           // transposed operands of the same
-    key_lane.init(32 - shift, lane);
-    key_tr.init(32 - shift, lane);
+    key_lane.init(0, lane);
+    key_tr.init(0, lane);
     qry_lane.init(0, lane);
     qry_tr.init(0, lane);
 
@@ -311,7 +314,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
             RowOperand<C> kop, vop;
-            const int off = (qt - i0 + vb) * LL::kTileBytes;
+            const int off = (qt - i0 + 1 + vb) * LL::kTileBytes;
             read_rows<C>(kop, k_lds + off, key_lane);
             read_rows<C>(vop, v_lds + off, key_lane);
             s[vb] = dot_rows_mma<DT, C>(kop, qop);
@@ -378,7 +381,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         for (int ct = 0; ct < CT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
-            LDS_PTR(char) blk = k_lds + (qt - i0 + vb) * LL::kTileBytes;
+            LDS_PTR(char) blk = k_lds + (qt - i0 + 1 + vb) * LL::kTileBytes;
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(blk + key_tr.off[ct]), db[vb], acc[ct]);
         }
@@ -505,7 +508,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
     auto kern = window_blocks(g) == 2 ? fused_bwd_kernel<DT, C, 2> : fused_bwd_kernel<DT, C, 3>;
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
-    const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 4), (sp.nt + 2) * 4 * 512);
+    const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + 2) * 4 * 512);
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
                        (kThreads + 32 + (drpb ? kWaves * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
