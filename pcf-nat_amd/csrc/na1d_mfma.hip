@@ -44,13 +44,23 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     const Rsrc qs = make_rsrc(q + in_off, qry_bytes), ks = make_rsrc(k + in_off, key_bytes);
     const Rsrc vs = make_rsrc(v + in_off, key_bytes), os = make_rsrc(out + out_off, T * outl.pitch);
     const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
+    const bool out_whole_lines = stores_whole_lines(outl.pitch, C, 0);
 
     // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
     {
         const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch);
-        stage_direct<C, MT + 2>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
-        stage_direct<C, MT>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-        stage_direct<C, MT + 2>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+        if (strips == 1 && (in.pitch == 2 * C || C % 64 == 0)) {      // nobody else reads these rows' lines
+            stage_direct<C, MT + 2, kReadOnce>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<C, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadOnce>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+        } else {
+            stage_direct<C, MT + 2, kReadShared>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+            if (in.pitch == 2 * C || C % 64 == 0)
+                stage_direct<C, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            else
+                stage_direct<C, MT, kReadShared>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadShared>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+        }
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
     }
 
@@ -145,7 +155,10 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
             u32x2 w;
             w.x = Mma<DT>::pack(o[ct][0] * inv, o[ct][1] * inv);
             w.y = Mma<DT>::pack(o[ct][2] * inv, o[ct][3] * inv);
-            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * outl.pitch + ct * 32 + g * 8, 0, 0);
+            if (out_whole_lines)
+                __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * outl.pitch + ct * 32 + g * 8, 0, kStoreAux);
+            else
+                __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * outl.pitch + ct * 32 + g * 8, 0, 0);
         }
         if (g == 0)
             __builtin_amdgcn_raw_buffer_store_b32(
@@ -273,10 +286,17 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch);
         // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * i0 - 16 + tid) * 4, 0, 0, 0);
-        stage_direct<C, MT + 1 + NBV>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-        stage_direct<C, MT + 2>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
-        stage_direct<C, MT + 1 + NBV>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-        stage_direct<C, MT + 2>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
+        if (strips == 1 && (in.pitch == 2 * C || C % 64 == 0) && (outl.pitch == 2 * C || C % 64 == 0)) {
+            stage_direct<C, MT + 1 + NBV, kReadOnce>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadOnce>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 1 + NBV, kReadOnce>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadOnce>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
+        } else {
+            stage_direct<C, MT + 1 + NBV, kReadShared>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadShared>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 1 + NBV, kReadShared>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadShared>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
+        }
         stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
     }
 
@@ -300,6 +320,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
     const Rsrc dqs = make_rsrc(dq + in_off, T * in.pitch);
+    const bool dq_whole_lines = stores_whole_lines(in.pitch, C, 0);
     u32x2 sc[TPW][2][2];                // [tile of this wave][X/Y slot set][P / dS], rounded to 16 bit
 #pragma unroll
     for (int jt = 0; jt < TPW; ++jt) {
@@ -390,7 +411,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             u32x2 w;
             w.x = Mma<DT>::pack(acc[ct][0] * scale, acc[ct][1] * scale);
             w.y = Mma<DT>::pack(acc[ct][2] * scale, acc[ct][3] * scale);
-            __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * in.pitch + ct * 32 + g * 8, 0, 0);
+            if (dq_whole_lines)
+                __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * in.pitch + ct * 32 + g * 8, 0, kStoreAux);
+            else
+                __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * in.pitch + ct * 32 + g * 8, 0, 0);
         }
     }
 
@@ -448,6 +472,9 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     const Rsrc dks = make_rsrc(dk + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
     const Rsrc dvs = make_rsrc(dv + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
     const int kp_lo = i0 + (shift == 16 ? 1 : 0), kp_hi = i1 - (shift == 0 ? 1 : 0);
+    // a key block starts `shift` rows before a tile (non-temporal stores of split lines cost cfg2's backward 5 %;
+    // where lines are whole they gain 10 %)
+    const bool whole_lines = stores_whole_lines(in.pitch, C, shift);
     for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
         f32x4 acck[CT], accv[CT];
 #pragma unroll
@@ -481,8 +508,13 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             wk.y = Mma<DT>::pack(acck[ct][2] * scale, acck[ct][3] * scale);
             wv.x = Mma<DT>::pack(accv[ct][0], accv[ct][1]);
             wv.y = Mma<DT>::pack(accv[ct][2], accv[ct][3]);
-            __builtin_amdgcn_raw_buffer_store_b64(wk, dks, row_off + ct * 32 + g * 8, 0, 0);
-            __builtin_amdgcn_raw_buffer_store_b64(wv, dvs, row_off + ct * 32 + g * 8, 0, 0);
+            if (whole_lines) {
+                __builtin_amdgcn_raw_buffer_store_b64(wk, dks, row_off + ct * 32 + g * 8, 0, kStoreAux);
+                __builtin_amdgcn_raw_buffer_store_b64(wv, dvs, row_off + ct * 32 + g * 8, 0, kStoreAux);
+            } else {
+                __builtin_amdgcn_raw_buffer_store_b64(wk, dks, row_off + ct * 32 + g * 8, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b64(wv, dvs, row_off + ct * 32 + g * 8, 0, 0);
+            }
         }
     }
 

@@ -98,6 +98,20 @@ __device__ inline Rsrc make_rsrc(const void *base, int bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, 0x00020000);
 }
 
+// Cache policy of the streaming accesses (the `aux` operand of the buffer builtins; bit 1 = nt, non-temporal).
+// Outputs are written once and rows that only one workgroup reads are read once: both are marked nt, which is
+// worth 10-15 % of a forward launch here.  Rows that a neighbouring strip reads again as its halo are loaded
+// with the default policy so that the second read hits L2 (marking them nt costs cfg2's forward 15 %).
+constexpr int kReadOnce = 2, kReadShared = 0, kStoreAux = 2;
+// A wave stores 16 rows of 2*C bytes starting `first_row` rows off a tile boundary.  The non-temporal policy
+// pays only when the wave's rows make up whole 128-byte lines by themselves: packed rows starting on a line, or
+// strided rows that are whole lines each.  Otherwise other waves (or other heads' workgroups) write the rest of
+// the lines later, and only the default policy lets L2 merge the pieces.
+__device__ inline bool stores_whole_lines(int pitch, int C, int first_row) {
+    if (pitch == 2 * C) return (first_row * pitch) % 128 == 0 && (16 * pitch) % 128 == 0;
+    return (2 * C) % 128 == 0 && pitch % 128 == 0;
+}
+
 // ---- LDS layout -------------------------------------------------------------------
 // Rows of C 16-bit channels, row-major and unpadded; the 16-byte units of a row
 // are XOR-swizzled with the row's 256-byte phase so that the 16 rows an operand
@@ -146,7 +160,7 @@ template <int C> __device__ inline int direct_lane_offset(int wave, int lane, in
     const int su = u % Lds<C>::kUnits;
     return (lane / Lds<C>::kUnits) * pitch + (su ^ Lds<C>::swz(u / Lds<C>::kUnits)) * 16;
 }
-template <int C, int NTILES>
+template <int C, int NTILES, int AUX>
 __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, int ntiles, int wave, int lane_off,
                                     int pitch = Lds<C>::kRowBytes) {
     constexpr int kRounds = (region_bytes<C>(NTILES) / kChunk + kWaves - 1) / kWaves;
@@ -157,7 +171,7 @@ __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, 
     for (int j = 0; j < kRounds; ++j) {
         const int c = j * kWaves + wave;
         if (c < chunks)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * kChunk), 16, base + c * step, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * kChunk), 16, base + c * step, 0, 0, AUX);
     }
 }
 __device__ inline void wait_direct() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }

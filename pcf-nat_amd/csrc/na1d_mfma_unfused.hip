@@ -26,7 +26,7 @@ __device__ inline void stage_scores(Rsrc src, int first, LDS_PTR(float) region, 
         const int c = j * kWaves + wave;
         if (c < chunks)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * (kChunk / 4)), 16,
-                                                     first * 4 + c * kChunk + lane * 16, 0, 0, 0);
+                                                     first * 4 + c * kChunk + lane * 16, 0, 0, kReadShared);
     }
 }
 
@@ -64,8 +64,8 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     {
         const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
         const int lane_off = direct_lane_offset<C>(wave, lane);
-        stage_direct<C, MT + 2>(make_rsrc(kb + seq_off, key_bytes), 16 * i0 - 16, k_lds, nt + 2, wave, lane_off);
-        stage_direct<C, MT>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off);
+        stage_direct<C, MT + 2, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * i0 - 16, k_lds, nt + 2, wave, lane_off);
+        stage_direct<C, MT, kReadShared>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off);
     }
     const Rsrc as = make_rsrc(attn + (int64_t)b * T * W, T * W * 4);
     RowLane<C> k_lane, q_lane;
@@ -95,8 +95,13 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         const int first = 16 * i * W;                             // floats into the sequence's score rows
-        for (int u = lane; u * 4 < 16 * W; u += 64)
-            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, 0);
+        if (W % 2 == 0) {       // a tile's 16*W floats are whole 128-byte lines: written once, by this wave alone
+            for (int u = lane; u * 4 < 16 * W; u += 64)
+                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, kStoreAux);
+        } else {                // neighbouring tiles share the first and last line: let L2 merge them
+            for (int u = lane; u * 4 < 16 * W; u += 64)
+                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, 0);
+        }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");    // tile read before the next one overwrites it
         __builtin_amdgcn_wave_barrier();
     }
@@ -130,7 +135,7 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
         const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C;
-        stage_direct<C, MT + 2>(make_rsrc(v + seq_off, key_bytes), 16 * i0 - 16, v_lds, nt + 2, wave,
+        stage_direct<C, MT + 2, kReadShared>(make_rsrc(v + seq_off, key_bytes), 16 * i0 - 16, v_lds, nt + 2, wave,
                                 direct_lane_offset<C>(wave, lane));
         stage_scores<C>(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, s_lds, nt, W, wave, lane);
     }
@@ -162,7 +167,7 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
             u32x2 w;
             w.x = Mma<DT>::pack(o[ct][0], o[ct][1]);
             w.y = Mma<DT>::pack(o[ct][2], o[ct][3]);
-            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * (2 * C) + ct * 32 + g * 8, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * (2 * C) + ct * 32 + g * 8, 0, kStoreAux);
         }
     }
 }
@@ -195,7 +200,7 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
         const int rows_hi = min(T, 16 * (i1 + 1));
-        stage_direct<C, MT + 2>(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * i0 - 16, x_lds, nt + 2, wave,
+        stage_direct<C, MT + 2, kReadShared>(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * i0 - 16, x_lds, nt + 2, wave,
                                 direct_lane_offset<C>(wave, lane));
         stage_scores<C>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), (16 * i0 - 16) * W, s_lds, nt + 2, W, wave, lane);
     }
@@ -231,7 +236,7 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
             u32x2 w;
             w.x = Mma<DT>::pack(acc[ct][0], acc[ct][1]);
             w.y = Mma<DT>::pack(acc[ct][2], acc[ct][3]);
-            __builtin_amdgcn_raw_buffer_store_b64(w, os, row_off + ct * 32 + g * 8, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(w, os, row_off + ct * 32 + g * 8, 0, kStoreAux);
         }
     }
 }
