@@ -12,14 +12,52 @@ import torch
 from . import _lib
 
 
+def _residue(x4, r, d):
+    """Rows r, r+d, r+2d, ... of a ``[N, H, T, C]`` view: the sub-sequence a dilated window lives in."""
+    return x4[:, :, r::d]
+
+
+def _residue_lengths(t_valid, r, d):
+    """Valid length of that sub-sequence: rows r + d*t' < t_valid."""
+    return None if t_valid is None else ((t_valid - r + d - 1) // d).clamp_(min=0).to(torch.int32)
+
+
+def _strided_or_packed_forward(out4, lse, q4, k4, v4, rpb, t_valid, W, left, scale):
+    """Forward on ``[N, H, T, C]`` views through the strided entry point, or - for shapes it does not cover -
+    on packed copies through the packed one.  Returns the packed output when it had to be made."""
+    if _lib.call_fused_forward_strided(out4, lse, q4, k4, v4, rpb, t_valid, W, left, scale) == 0:
+        return None
+    N, H, T, C = q4.shape
+    qp, kp, vp = (z.contiguous().view(N * H, T, C) for z in (q4, k4, v4))
+    op = torch.empty_like(qp)
+    _lib.call_fused_forward(op, lse, qp, kp, vp, rpb, t_valid, N * H, H, T, C, W, left, scale)
+    out4.copy_(op.view(N, H, T, C))
+    return op
+
+
+def _strided_or_packed_backward(dq4, dk4, dv4, drpb, q4, k4, v4, packed_out, dout4, lse, rpb, t_valid, W, left, scale, ws):
+    if packed_out is None:
+        st = _lib.call_fused_backward_strided(dq4, dk4, dv4, drpb, q4, k4, v4, dout4, lse, rpb, t_valid, W, left, scale,
+                                              workspace=ws)
+        assert st == 0
+        return
+    N, H, T, C = q4.shape
+    qp, kp, vp, gp = (z.contiguous().view(N * H, T, C) for z in (q4, k4, v4, dout4))
+    dqp, dkp, dvp = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
+    _lib.call_fused_backward(dqp, dkp, dvp, drpb, qp, kp, vp, packed_out, gp, lse, rpb, t_valid, N * H, H, T, C, W, left,
+                             scale, workspace=ws)
+    for dst, src in ((dq4, dqp), (dk4, dkp), (dv4, dvp)):
+        dst.copy_(src.view(N, H, T, C))
+
+
 class _FusedNA1D(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, rpb, t_valid, num_heads, win_size, left, scale, deterministic):
+    def forward(ctx, q, k, v, rpb, t_valid, num_heads, win_size, left, scale, deterministic, dilation):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
         assert q.dtype == k.dtype == v.dtype
         assert q.dim() == 3 and q.shape == k.shape == v.shape, "q, k, v must all be [B, T, C]"
         B, T, C = q.shape
-        assert B % num_heads == 0
+        assert B % num_heads == 0 and dilation >= 1
         ctx.rpb_shape = None if rpb is None else rpb.shape
         if rpb is not None:
             rpb = rpb.detach().reshape(num_heads, win_size).to(torch.float32).contiguous()
@@ -27,16 +65,31 @@ class _FusedNA1D(torch.autograd.Function):
             assert t_valid.numel() == B // num_heads
             t_valid = t_valid.to(device=q.device, dtype=torch.int32).contiguous()
         out = torch.empty_like(q)
-        lse = torch.empty((B, T), dtype=torch.float32, device=q.device)
-        _lib.call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, num_heads, T, C, win_size, left, scale)
-        ctx.save_for_backward(q, k, v, out, lse, rpb, t_valid)
-        ctx.geom = (num_heads, win_size, left, scale, deterministic)
+        ctx.geom = (num_heads, win_size, left, scale, deterministic, dilation)
+        if dilation == 1:
+            lse = torch.empty((B, T), dtype=torch.float32, device=q.device)
+            _lib.call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, num_heads, T, C, win_size, left, scale)
+            ctx.save_for_backward(q, k, v, out, rpb, t_valid, lse)
+            return out
+        # Dilation d: slot j of row t is row t + (j - left) * d, so the rows of one residue class t mod d only
+        # ever meet each other - d independent, undilated problems on every d-th row, read and written in place.
+        shape4 = (B // num_heads, num_heads, T, C)
+        q4, k4, v4, o4 = (z.view(shape4) for z in (q, k, v, out))
+        lses, ctx.packed_outs = [], []
+        for r in range(min(dilation, T)):
+            qr = _residue(q4, r, dilation)
+            lse = torch.empty((B, qr.shape[2]), dtype=torch.float32, device=q.device)
+            ctx.packed_outs.append(_strided_or_packed_forward(
+                _residue(o4, r, dilation), lse, qr, _residue(k4, r, dilation), _residue(v4, r, dilation), rpb,
+                _residue_lengths(t_valid, r, dilation), win_size, left, scale))
+            lses.append(lse)
+        ctx.save_for_backward(q, k, v, out, rpb, t_valid, *lses)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, out, lse, rpb, t_valid = ctx.saved_tensors
-        num_heads, win_size, left, scale, deterministic = ctx.geom
+        q, k, v, out, rpb, t_valid, *lses = ctx.saved_tensors
+        num_heads, win_size, left, scale, deterministic, dilation = ctx.geom
         B, T, C = q.shape
         dout = dout.contiguous()
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
@@ -44,17 +97,26 @@ class _FusedNA1D(torch.autograd.Function):
         if rpb is not None and ctx.needs_input_grad[3]:
             drpb = torch.zeros((num_heads, win_size), dtype=torch.float32, device=q.device)
             if deterministic:   # fold the per-workgroup partial sums in a fixed order instead of with atomics
-                nbytes = _lib.fused_backward_workspace_bytes(B, num_heads, T, C, win_size, left, q.dtype)
+                nbytes = _lib.fused_backward_workspace_bytes(B, num_heads, -(-T // dilation), C, win_size, left, q.dtype)
                 if nbytes > 0:
                     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-        _lib.call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid,
-                                 B, num_heads, T, C, win_size, left, scale, workspace=ws)
+        if dilation == 1:
+            _lib.call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lses[0], rpb, t_valid,
+                                     B, num_heads, T, C, win_size, left, scale, workspace=ws)
+        else:
+            shape4 = (B // num_heads, num_heads, T, C)
+            views = [z.view(shape4) for z in (dq, dk, dv, q, k, v, dout)]
+            for r, lse in enumerate(lses):
+                a = [_residue(z, r, dilation) for z in views]
+                _strided_or_packed_backward(a[0], a[1], a[2], drpb, a[3], a[4], a[5], ctx.packed_outs[r], a[6], lse, rpb,
+                                            _residue_lengths(t_valid, r, dilation), win_size, left, scale, ws)
         if drpb is not None:
             drpb = drpb.view(ctx.rpb_shape)
-        return dq, dk, dv, drpb, None, None, None, None, None, None
+        return dq, dk, dv, drpb, None, None, None, None, None, None, None
 
 
-def na1d_fused(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, scale=1.0, deterministic=False):
+def na1d_fused(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, scale=1.0, deterministic=False,
+               dilation=1):
     """Fused neighbourhood attention.
 
     q, k, v : contiguous ``[B, T, C]`` bf16/fp16, ``B = N * num_heads``.  ``q`` is
@@ -66,9 +128,12 @@ def na1d_fused(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, sca
               atomics by default (fast, last bits vary from run to run); ``True``
               folds the partial sums in a fixed order through a scratch buffer.
               dq, dk, dv never use atomics.
+    dilation : window slot j of row t addresses row ``t + (j - left) * dilation`` (the reference computes this on
+              the CPU only, models/PCF_NATransformer.py:101-116,158-170; its CUDA path asserts dilation == 1).
     Returns ``[B, T, C]`` in q's dtype.  The gradient of ``rpb`` has rpb's shape.
     """
-    return _FusedNA1D.apply(q, k, v, rpb, t_valid, num_heads, win_size, left, float(scale), bool(deterministic))
+    return _FusedNA1D.apply(q, k, v, rpb, t_valid, num_heads, win_size, left, float(scale), bool(deterministic),
+                            int(dilation))
 
 
 def na1d_fused_forward_lse(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, scale=1.0):
@@ -88,8 +153,8 @@ class _FusedNA1DQKV(torch.autograd.Function):
     """Fused NA1D straight on the qkv projection's output ``[N, T, 3, H, C]`` -> ``[N, T, H*C]``."""
 
     @staticmethod
-    def forward(ctx, qkv, rpb, t_valid, win_size, left, scale, deterministic):
-        assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.is_contiguous()
+    def forward(ctx, qkv, rpb, t_valid, win_size, left, scale, deterministic, dilation):
+        assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.is_contiguous() and dilation >= 1
         N, T, _, H, C = qkv.shape
         ctx.rpb_shape = None if rpb is None else rpb.shape
         if rpb is not None:
@@ -97,56 +162,47 @@ class _FusedNA1DQKV(torch.autograd.Function):
         if t_valid is not None:
             assert t_valid.numel() == N
             t_valid = t_valid.to(device=qkv.device, dtype=torch.int32).contiguous()
-        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))          # [N, H, T, C] views
+        q4, k4, v4 = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))       # [N, H, T, C] views
         out = torch.empty((N, T, H, C), dtype=qkv.dtype, device=qkv.device)
-        lse = torch.empty((N * H, T), dtype=torch.float32, device=qkv.device)
-        st = _lib.call_fused_forward_strided(out.permute(0, 2, 1, 3), lse, q, k, v, rpb, t_valid, win_size, left, scale)
-        ctx.strided = st == 0
-        ctx.packed_out = None
-        if not ctx.strided:      # shape outside the strided kernels: pack, as the reference does, and use the packed op
-            qp, kp, vp = (z.contiguous().view(N * H, T, C) for z in (q, k, v))
-            op = torch.empty_like(qp)
-            _lib.call_fused_forward(op, lse, qp, kp, vp, rpb, t_valid, N * H, H, T, C, win_size, left, scale)
-            out.copy_(op.view(N, H, T, C).permute(0, 2, 1, 3))
-            ctx.packed_out = op          # the generic backward kernel reads it
-        ctx.save_for_backward(qkv, lse, rpb, t_valid)
-        ctx.geom = (win_size, left, scale, deterministic)
+        o4 = out.permute(0, 2, 1, 3)
+        lses, ctx.packed_outs = [], []
+        for r in range(min(dilation, T)):                                         # see _FusedNA1D.forward
+            qr = _residue(q4, r, dilation)
+            lse = torch.empty((N * H, qr.shape[2]), dtype=torch.float32, device=qkv.device)
+            ctx.packed_outs.append(_strided_or_packed_forward(
+                _residue(o4, r, dilation), lse, qr, _residue(k4, r, dilation), _residue(v4, r, dilation), rpb,
+                _residue_lengths(t_valid, r, dilation), win_size, left, scale))
+            lses.append(lse)
+        ctx.save_for_backward(qkv, rpb, t_valid, *lses)
+        ctx.geom = (win_size, left, scale, deterministic, dilation)
         return out.view(N, T, H * C)
 
     @staticmethod
     def backward(ctx, dout):
-        qkv, lse, rpb, t_valid = ctx.saved_tensors
-        win_size, left, scale, deterministic = ctx.geom
+        qkv, rpb, t_valid, *lses = ctx.saved_tensors
+        win_size, left, scale, deterministic, dilation = ctx.geom
         N, T, _, H, C = qkv.shape
-        dout = dout.contiguous().view(N, T, H, C)
+        g4 = dout.contiguous().view(N, T, H, C).permute(0, 2, 1, 3)
         dqkv = torch.empty_like(qkv)
         drpb = ws = None
         if rpb is not None and ctx.needs_input_grad[1]:
             drpb = torch.zeros((H, win_size), dtype=torch.float32, device=qkv.device)
             if deterministic:
-                nbytes = _lib.fused_backward_workspace_bytes(N * H, H, T, C, win_size, left, qkv.dtype)
+                nbytes = _lib.fused_backward_workspace_bytes(N * H, H, -(-T // dilation), C, win_size, left, qkv.dtype)
                 if nbytes > 0:
                     ws = torch.empty(nbytes, dtype=torch.uint8, device=qkv.device)
-        q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
-        if ctx.strided:
-            dq, dk, dv = (dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
-            st = _lib.call_fused_backward_strided(dq, dk, dv, drpb, q, k, v, dout.permute(0, 2, 1, 3), lse, rpb, t_valid,
-                                                  win_size, left, scale, workspace=ws)
-            assert st == 0
-        else:
-            qp, kp, vp = (z.contiguous().view(N * H, T, C) for z in (q, k, v))
-            gp = dout.permute(0, 2, 1, 3).contiguous().view(N * H, T, C)
-            dqp, dkp, dvp = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
-            _lib.call_fused_backward(dqp, dkp, dvp, drpb, qp, kp, vp, ctx.packed_out, gp, lse, rpb, t_valid, N * H, H, T, C,
-                                     win_size, left, scale, workspace=ws)
-            for i, z in enumerate((dqp, dkp, dvp)):
-                dqkv[:, :, i].copy_(z.view(N, H, T, C).permute(0, 2, 1, 3))
+        views = [dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)] + [qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)]
+        for r, lse in enumerate(lses):
+            a = [_residue(z, r, dilation) for z in views]
+            _strided_or_packed_backward(a[0], a[1], a[2], drpb, a[3], a[4], a[5], ctx.packed_outs[r],
+                                        _residue(g4, r, dilation), lse, rpb, _residue_lengths(t_valid, r, dilation),
+                                        win_size, left, scale, ws)
         if drpb is not None:
             drpb = drpb.view(ctx.rpb_shape)
-        return dqkv, drpb, None, None, None, None, None
+        return dqkv, drpb, None, None, None, None, None, None
 
 
-def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deterministic=False):
+def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deterministic=False, dilation=1):
     """Fused neighbourhood attention on a token-major qkv projection output.
 
     qkv : contiguous ``[N, T, 3, H, C]`` bf16/fp16 (the ``[N, T, 3*dim]`` output of the projection, viewed).
@@ -156,4 +212,4 @@ def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deter
           reference multiplies q by it in 16 bit beforehand).
     Other arguments as in :func:`na1d_fused`.
     """
-    return _FusedNA1DQKV.apply(qkv, rpb, t_valid, win_size, left, float(scale), bool(deterministic))
+    return _FusedNA1DQKV.apply(qkv, rpb, t_valid, win_size, left, float(scale), bool(deterministic), int(dilation))

@@ -208,6 +208,44 @@ def test_fused_on_projection_layout_matches_oracle_and_packed_operator(geom, dty
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", [(2, 4, 61, 16, 27, 13, 2), (3, 2, 50, 32, 15, 7, 3), (2, 2, 40, 64, 7, 3, 4),
+                                  (2, 3, 33, 24, 8, 3, 2), (1, 2, 5, 16, 5, 2, 7), (2, 2, 100, 16, 9, 0, 5)],
+                         ids=lambda g: "x".join(map(str, g)))
+def test_dilated_windows_match_oracle(geom, dtype):
+    """dilation > 1 (CPU-only in the reference, models/PCF_NATransformer.py:101-116,158-170): slot j of row t is
+    row t + (j - left) * d; packed and projection-layout operators, with rpb and per-sample valid lengths."""
+    N, H, T, C, W, L, D = geom
+    g = torch.Generator().manual_seed(21)
+    qkv = (torch.randn(N, T, 3, H, C, generator=g) * (C ** -0.25)).to(dtype)
+    do = torch.randn(N, T, H * C, generator=g).to(dtype)
+    rpb = torch.randn(H, W, generator=g) * 0.5
+    pad = torch.tensor([0, T // 3, T - 1][:N] + [1] * max(0, N - 3))
+    t_valid = (T - pad).to(torch.int32).cuda()
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3).contiguous().view(N * H, T, C) for i in range(3))
+    dop = do.view(N, T, H, C).permute(0, 2, 1, 3).contiguous().view(N * H, T, C)
+    want_o, _, _ = O.na1d_forward(q.float(), k.float(), v.float(), W, L, rpb, pad, H, dilation=D)
+    wq, wk, wv, wr = O.na1d_backward(q.float(), k.float(), v.float(), dop.float(), W, L, rpb, pad, H, dilation=D)
+    tol = TOL[dtype]
+
+    qd, kd, vd = (z.cuda().requires_grad_(True) for z in (q, k, v))
+    rd = rpb.cuda().requires_grad_(True)
+    out = na1d_fused(qd, kd, vd, W, L, rpb=rd, t_valid=t_valid, num_heads=H, dilation=D)
+    out.backward(dop.cuda())
+    assert O.rel_l2(out.float(), want_o) < tol, "O"
+    for name, got, want in (("dQ", qd.grad, wq), ("dK", kd.grad, wk), ("dV", vd.grad, wv)):
+        assert O.rel_l2(got.float(), want) < tol, name
+    assert _err(rd.grad, wr) < tol, "drpb"
+
+    xd = qkv.cuda().requires_grad_(True)
+    out2 = na1d_fused_qkv(xd, W, L, rpb=rpb.cuda(), t_valid=t_valid, dilation=D)
+    out2.backward(do.cuda())
+    unpack = lambda z: z.reshape(N, H, T, C).permute(0, 2, 1, 3)
+    assert torch.equal(out2.view(N, T, H, C), unpack(out))
+    for i, z in enumerate((qd, kd, vd)):
+        assert torch.equal(xd.grad[:, :, i], unpack(z.grad))
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
 def test_strided_entry_points_leave_the_gaps_alone(dtype):
     """Rows 3*H*C apart with the k and v slots (and a pad column) between them: nothing but the addressed
     rows may be written."""
