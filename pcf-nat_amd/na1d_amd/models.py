@@ -50,8 +50,12 @@ class BatchNorm1d(nn.BatchNorm1d):
     off the memory roofline at these shapes ([256, 256, 100] bf16 measured 98 us there, 21 us here)."""
 
     def forward(self, x):
-        with torch.backends.cudnn.flags(enabled=False):
+        was = torch.backends.cudnn.enabled
+        torch.backends.cudnn.enabled = False
+        try:
             return super().forward(x)
+        finally:
+            torch.backends.cudnn.enabled = was
 
 
 class Conv1x1(nn.Conv1d):
@@ -260,7 +264,7 @@ class NAttention(nn.Module):
     """Neighbourhood attention layer (PCF_NATransformer.py:44-178 / MFA_NATransformer.py:43-177)."""
 
     def __init__(self, frames, dim, num_heads, win_size, groups=1, channels_first=True, dtype=torch.bfloat16,
-                 na="fused"):
+                 na="fused", dilation=1):
         super().__init__()
         if isinstance(win_size, int):
             assert win_size > 0
@@ -271,15 +275,15 @@ class NAttention(nn.Module):
         head_dim = dim // num_heads
         assert dim % num_heads == 0 and head_dim % 8 == 0
         self.win_size, self.left, self.dim, self.num_heads, self.groups = win_size, left, dim, num_heads, groups
-        self.channels_first, self.na = channels_first, na
+        self.channels_first, self.na, self.dilation = channels_first, na, dilation
         self.scale = head_dim ** -0.5
         self.qkv = _Projection.make(dim, dim * 3, True, groups, channels_first)
         self.relative_position_bias = nn.Parameter(torch.zeros(1, num_heads, 1, win_size))
         nn.init.normal_(self.relative_position_bias, mean=0.0, std=0.02)
         self.proj = _Projection.make(dim, dim, True, groups, channels_first)
         self.register_buffer("attn_mask", _window_mask(frames, win_size, left, None, torch.float32, "cpu").unsqueeze(1))
-        if na == "unfused":
-            self.NA1d_QK_Function, self.NA1d_AV_Function = getNA1dFunction(C=head_dim, dilation=1, dtype=dtype)
+        if na == "unfused":     # like the reference's CUDA path, the two-call chain has no dilated kernels
+            self.NA1d_QK_Function, self.NA1d_AV_Function = getNA1dFunction(C=head_dim, dilation=dilation, dtype=dtype)
 
     def forward(self, x, padding=None):
         n = x.shape[0]
@@ -290,10 +294,11 @@ class NAttention(nn.Module):
             return self._forward_token_major(x, n, t, t_valid)
         q, k, v = _split_heads(self.qkv(x), h, self.groups, self.channels_first)
         q = q * self.scale                                   # in the activation dtype, as the reference does (:141)
+        extra = {} if self.dilation == 1 else {"dilation": self.dilation}
         if callable(self.na):
-            out = self.na(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h)
+            out = self.na(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h, **extra)
         elif self.na == "fused":
-            out = na1d_fused(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h)
+            out = na1d_fused(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h, **extra)
         else:                                                # the reference's un-fused chain (:141-150)
             attn = self.NA1d_QK_Function.apply(q, k, w, left, 1).view(n, h, t, w)
             attn = attn + self.relative_position_bias
@@ -315,7 +320,8 @@ class NAttention(nn.Module):
         else:
             qkv = self.qkv(x)
         out = na1d_fused_qkv(qkv.view(n, t, 3, h, self.dim // h), self.win_size, self.left,
-                             rpb=self.relative_position_bias, t_valid=t_valid, scale=self.scale)      # [N, T, dim]
+                             rpb=self.relative_position_bias, t_valid=t_valid, scale=self.scale,
+                             dilation=self.dilation)                                                  # [N, T, dim]
         if self.channels_first:
             wp, bp = _prepared(self.proj, "dense", out, lambda: (_dense_weight(self.proj), self.proj.bias))
             return torch.bmm(wp.unsqueeze(0).expand(n, -1, -1), out.transpose(1, 2)).add_(bp.view(1, -1, 1))  # [N, dim, T]
@@ -339,10 +345,13 @@ class GlobalAttention(nn.Module):
         q, k, v = _split_heads(self.qkv(x), self.num_heads, self.groups, self.channels_first)
         t, hd = q.shape[1], q.shape[2]
         q, k, v = (z.view(n, self.num_heads, t, hd) for z in (q, k, v))
-        attn = (q * self.scale) @ k.transpose(-2, -1)
-        if attn_mask is not None:
-            attn = attn + attn_mask
-        out = torch.softmax(attn, dim=-1) @ v
+        if x.device.type == "cuda":      # one library kernel instead of matmul -> mask -> softmax -> matmul
+            out = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, scale=self.scale)
+        else:
+            attn = (q * self.scale) @ k.transpose(-2, -1)
+            if attn_mask is not None:
+                attn = attn + attn_mask
+            out = torch.softmax(attn, dim=-1) @ v
         return self.proj(_merge_heads(out.reshape(n * self.num_heads, t, hd), n, self.num_heads, self.channels_first))
 
 
@@ -360,12 +369,14 @@ class Mlp(nn.Module):
 class NATFLayer(nn.Module):
     """norm -> attention -> residual; norm -> MLP -> residual (PCF :228-265)."""
 
-    def __init__(self, frames, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na, mlp_ratio=4):
+    def __init__(self, frames, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na, mlp_ratio=4,
+                 dilation=1):
         super().__init__()
         self.local = isinstance(win_size, list) or win_size > 0
         if self.local:
-            self.attn = NAttention(frames, dim, num_heads, win_size, groups, channels_first, dtype, na)
+            self.attn = NAttention(frames, dim, num_heads, win_size, groups, channels_first, dtype, na, dilation)
         else:
+            assert dilation == 1
             self.attn = GlobalAttention(dim, num_heads, groups, channels_first)
         norm = BatchNorm1d if channels_first else TokenBatchNorm
         self.norm1 = norm(dim)
@@ -382,13 +393,13 @@ class NATFLayer(nn.Module):
 
 class NATFBlock(nn.Module):
     def __init__(self, frames, depth, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na,
-                 use_checkpoint=False):
+                 use_checkpoint=False, dilation=1):
         super().__init__()
         pick = lambda v, i: v[i] if isinstance(v, list) else v
         self.use_checkpoint = use_checkpoint if isinstance(use_checkpoint, list) else [use_checkpoint] * depth
         self.blocks = nn.ModuleList([
             NATFLayer(frames, dim, pick(num_heads, i), pick(win_size, i), pick(groups, i), pick(drop_path, i),
-                      channels_first, dtype, na) for i in range(depth)])
+                      channels_first, dtype, na, dilation=pick(dilation, i)) for i in range(depth)])
 
     def forward(self, x, padding=None, pos_emb=None, attn_mask_global=None):
         for layer, ckpt in zip(self.blocks, self.use_checkpoint):
@@ -415,7 +426,8 @@ class PatchEmbed(nn.Module):
 class _NATransformer(nn.Module):
     def __init__(self, channels_first, frames=300, patch_size=2, in_chans=80, output_emb_size=192, embed_dim=256,
                  depths=(4, 4, 4, 4), num_heads=None, win_size=None, groups=(8, 4, 2, 1), drop_path_rate=0.0,
-                 proj_channel=1536, asp=True, poolnorm=True, use_checkpoint=False, dtype=torch.bfloat16, na="fused"):
+                 proj_channel=1536, asp=True, poolnorm=True, use_checkpoint=False, dtype=torch.bfloat16, na="fused",
+                 dilation=1):
         super().__init__()
         depths = list(depths)
         nb = len(depths)
@@ -437,7 +449,7 @@ class _NATransformer(nn.Module):
         self.blocks = nn.ModuleList([
             NATFBlock(emb_frames, depths[i], embed_dim, pick(num_heads, i), pick(win_size, i),
                       pick(groups, i) if channels_first else 1, dpr[sum(depths[:i]):sum(depths[:i + 1])],
-                      channels_first, dtype, na, pick(use_checkpoint, i)) for i in range(nb)])
+                      channels_first, dtype, na, pick(use_checkpoint, i), pick(dilation, i)) for i in range(nb)])
         self.norm = BatchNorm1d(embed_dim * nb)
         self.proj = TDNNBlock(embed_dim * nb, proj_channel, 1)
         self.pool = AttentiveStatisticsPooling(proj_channel) if asp else StatisticsPooling()

@@ -10,10 +10,10 @@ from na1d_amd import models
 pytestmark = pytest.mark.gpu
 
 
-def oracle_na(q, k, v, W, L, rpb=None, t_valid=None, num_heads=1):
+def oracle_na(q, k, v, W, L, rpb=None, t_valid=None, num_heads=1, dilation=1):
     T = q.shape[1]
     pad = None if t_valid is None else (T - t_valid).to(torch.int64)
-    return O.na1d_forward(q, k, v, W, L, rpb.reshape(num_heads, W), pad, num_heads)[0]
+    return O.na1d_forward(q, k, v, W, L, rpb.reshape(num_heads, W), pad, num_heads, dilation=dilation)[0]
 
 
 def _randomise_norm_stats(model, seed):
@@ -48,6 +48,27 @@ def test_pcf_nat_4x4_inference_bf16(na):
             got = gpu(x.cuda())
     cos = F.cosine_similarity(got.float().cpu(), want, dim=-1)
     assert got.shape == (8, 192)
+    assert cos.min().item() >= 0.999, cos
+
+
+@pytest.mark.parametrize("na", ["fused", "fused_qkv"])
+def test_dilated_pcf_nat_bf16(na):
+    """The dilation argument of the model (models/PCF_NATransformer.py:323,333,373: an int or one per block),
+    which the reference can only run on the CPU: per-layer dilations 1..3 (1 for the global layers) and
+    variable lengths."""
+    kw = dict(dilation=[[2, 1], 2, [3, 1], [2, 3]], depths=(2, 2, 2, 2))
+    cpu = _twin(models.PCF_NATransformer, torch.bfloat16, **kw).eval()
+    gpu = models.PCF_NATransformer(na=na, dtype=torch.bfloat16, **kw)
+    gpu.load_state_dict(cpu.state_dict())
+    gpu = gpu.cuda().eval()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(4, 80, 240, generator=g)
+    lens = torch.tensor([1.0, 0.8, 0.55, 0.9])
+    with torch.no_grad():
+        want = cpu(x, lens)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            got = gpu(x.cuda(), lens.cuda())
+    cos = F.cosine_similarity(got.float().cpu(), want, dim=-1)
     assert cos.min().item() >= 0.999, cos
 
 
