@@ -21,13 +21,12 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
                    in.sample, in.head, in.pitch, outl.sample, outl.head, outl.pitch);
     // dynamic LDS (launch_fwd): K and V regions of nt+2 tiles starting one tile before the strip (row 16*i0 - 16:
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
-    // forward is not short of LDS), Q region of nt tiles, 32 bias floats
+    // forward is not short of LDS), Q region of nt tiles
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
     LDS_PTR(char) q_lds = v_lds + key_region;
-    LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + region_bytes<C>(nt));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -61,8 +60,11 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
                 stage_direct<C, MT, kReadShared>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
             stage_direct<C, MT + 2, kReadShared>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
         }
-        stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
     }
+
+    Window<NBV> win;
+    float rpb_raw[8];
+    make_window<NBV>(win, rpb_raw, rpb ? rpb + head * W : nullptr, W, L, shift, g, n);
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
@@ -76,9 +78,8 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     v_lane.init(16 - shift, lane);
 
     wait_direct();
+    add_bias<NBV>(win, rpb_raw);
     __syncthreads();
-    Window<NBV> win;
-    make_window<NBV>(win, bias_lds, W, L, shift, g, n);
 
     for (int i = i0 + wave; i < i1; i += kWaves) {
         const int tile_bytes = (i - i0) * LL::kTileBytes;
@@ -172,7 +173,7 @@ int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
     auto kern = window_blocks(g) == 2 ? fused_fwd_kernel<DT, C, 2> : fused_fwd_kernel<DT, C, 3>;
-    const size_t lds = (size_t)2 * region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt) + 32 * sizeof(float);
+    const size_t lds = (size_t)2 * region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                                                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
@@ -255,7 +256,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // dynamic LDS (see launch_bwd): [K region | V region] of nt+1+NBV tiles each, starting at the first key of
     // query tile i0-1 (row 16*(i0-1) - shift, so that virtual key blocks are whole tiles of the region), reused after
     // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt+2 tiles (rows 16*i0 - 16 ...); lse
-    // of the query-side rows; 32 bias floats; and - only when d rpb is wanted - 32 slot sums per wave
+    // of the query-side rows; and - only when d rpb is wanted - 32 slot sums per wave
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = region_bytes<C>(nt + 1 + NBV), qry_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
@@ -264,8 +265,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     LDS_PTR(char) q_lds = k_lds + kv_bytes;
     LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
     LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
-    LDS_PTR(float) bias_lds = lse_lds + kThreads;
-    LDS_PTR(float) rsum = bias_lds + 32;           // [kWaves][32] d rpb slot sums per wave
+    LDS_PTR(float) rsum = lse_lds + kThreads;      // [kWaves][32] d rpb slot sums per wave
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -297,8 +297,11 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             stage_direct<C, MT + 1 + NBV, kReadShared>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
             stage_direct<C, MT + 2, kReadShared>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
         }
-        stage_bias(bias_lds, rpb ? rpb + head * W : nullptr, W, tid);
     }
+
+    Window<NBV> win;
+    float rpb_raw[8];
+    make_window<NBV>(win, rpb_raw, rpb ? rpb + head * W : nullptr, W, L, shift, g, n);
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
@@ -313,9 +316,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     qry_tr.init(0, lane);
 
     wait_direct();
+    add_bias<NBV>(win, rpb_raw);
     __syncthreads();
-    Window<NBV> win;
-    make_window<NBV>(win, bias_lds, W, L, shift, g, n);
 
     // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
@@ -542,7 +544,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
     const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + 2) * 4 * 512);
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
-                       (kThreads + 32 + (drpb ? kWaves * 32 : 0)) * sizeof(float);
+                       (kThreads + (drpb ? kWaves * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                                                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb,

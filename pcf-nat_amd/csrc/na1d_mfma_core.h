@@ -271,34 +271,36 @@ template <int NBV> struct Window {
     u32x2 keep0, keep2;           // NBV 3: 16-bit lane masks that split packed X into blocks 0 and 2
 };
 
-// `bias_lds` holds this head's rpb row times log2(e) in slots [0, W) (zeros without
-// rpb); it is filled by stage_bias() before the workgroup barrier.
-__device__ inline void stage_bias(LDS_PTR(float) bias_lds, const float *rpb_h, int W, int tid) {
-    if (tid < 32) bias_lds[tid] = (rpb_h && tid < W) ? rpb_h[tid] * kLog2e : 0.f;
-}
-__device__ inline float bias_at(LDS_PTR(float) bias_lds, int j, int W) {   // -inf outside the band
-    const float val = bias_lds[j & 31];
-    return (j >= 0 && j < W) ? val : kNegInf;
-}
-
+// Window slots and bias of a lane.  The 8 rpb entries a lane needs are fetched with buffer loads issued
+// BEFORE the strip copies (they are tiny, hit L2, and have long arrived when the copies have; a NULL rpb makes an
+// empty resource, which reads as zeros), so nothing of this is left to do after the workgroup barrier but one
+// multiply-add per slot: bias = raw * log2(e) + (0 inside the band, -inf outside).
 template <int NBV>
-__device__ inline void make_window(Window<NBV> &w, LDS_PTR(float) bias_lds, int W, int L, int shift, int g, int n) {
+__device__ inline void make_window(Window<NBV> &w, float (&raw)[8], const float *rpb_h, int W, int L, int shift, int g,
+                                   int n) {
+    const Rsrc rs = make_rsrc(rpb_h, rpb_h ? W * 4 : 0);
     uint32_t m[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int j0 = 4 * g + r - shift - n + L;
-        w.bias_y[r] = bias_at(bias_lds, j0 + 16, W);
-        if (NBV == 2) {
-            w.from0[r] = true;
-            w.bias_x[r] = bias_at(bias_lds, j0, W);
-        } else {
-            w.from0[r] = j0 >= 0;
-            w.bias_x[r] = bias_at(bias_lds, w.from0[r] ? j0 : j0 + 32, W);
-        }
+        w.from0[r] = NBV == 2 || j0 >= 0;
+        const int jx = w.from0[r] ? j0 : j0 + 32, jy = j0 + 16;
+        raw[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, jx * 4, 0, 0));       // outside [0, W): 0
+        raw[4 + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, jy * 4, 0, 0));
+        w.bias_x[r] = (jx >= 0 && jx < W) ? 0.f : kNegInf;
+        w.bias_y[r] = (jy >= 0 && jy < W) ? 0.f : kNegInf;
         m[r] = w.from0[r] ? 0xffffu : 0u;
     }
     w.keep0 = u32x2{m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
     w.keep2 = u32x2{~w.keep0.x, ~w.keep0.y};
+}
+template <int NBV>
+__device__ inline void add_bias(Window<NBV> &w, const float (&raw)[8]) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        w.bias_x[r] = __builtin_fmaf(raw[r], kLog2e, w.bias_x[r]);
+        w.bias_y[r] = __builtin_fmaf(raw[4 + r], kLog2e, w.bias_y[r]);
+    }
 }
 
 // Kernel arguments live in memory and the compiler fetches each one next to its
