@@ -151,16 +151,10 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         }
 
         // rows past T fall outside the buffer and are dropped by the store
+        u32x2 ow[CT];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            u32x2 w;
-            w.x = Mma<DT>::pack(o[ct][0] * inv, o[ct][1] * inv);
-            w.y = Mma<DT>::pack(o[ct][2] * inv, o[ct][3] * inv);
-            if (out_whole_lines)
-                __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * outl.pitch + ct * 32 + g * 8, 0, kStoreAux);
-            else
-                __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * outl.pitch + ct * 32 + g * 8, 0, 0);
-        }
+        for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
+        store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines);
         if (g == 0)
             __builtin_amdgcn_raw_buffer_store_b32(
                 __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2), ls, qrow * 4, 0, 0);
@@ -408,16 +402,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(blk + key_tr.off[ct]), db[vb], acc[ct]);
         }
+        u32x2 qw[CT];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            u32x2 w;
-            w.x = Mma<DT>::pack(acc[ct][0] * scale, acc[ct][1] * scale);
-            w.y = Mma<DT>::pack(acc[ct][2] * scale, acc[ct][3] * scale);
-            if (dq_whole_lines)
-                __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * in.pitch + ct * 32 + g * 8, 0, kStoreAux);
-            else
-                __builtin_amdgcn_raw_buffer_store_b64(w, dqs, qrow * in.pitch + ct * 32 + g * 8, 0, 0);
-        }
+        for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[ct], scale);
+        store_tile<C>(dqs, qrow * in.pitch, qw, g, dq_whole_lines);
     }
 
     // d rpb: the window slot of each of a lane's 8 score registers is the same for every tile, so the lane
@@ -503,21 +491,14 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             }
         }
         const int row_off = (16 * (kp - i0) - shift + n) * in.pitch;    // outside the strip -> dropped
+        u32x2 kw[CT], vw[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            u32x2 wk, wv;
-            wk.x = Mma<DT>::pack(acck[ct][0] * scale, acck[ct][1] * scale);
-            wk.y = Mma<DT>::pack(acck[ct][2] * scale, acck[ct][3] * scale);
-            wv.x = Mma<DT>::pack(accv[ct][0], accv[ct][1]);
-            wv.y = Mma<DT>::pack(accv[ct][2], accv[ct][3]);
-            if (whole_lines) {
-                __builtin_amdgcn_raw_buffer_store_b64(wk, dks, row_off + ct * 32 + g * 8, 0, kStoreAux);
-                __builtin_amdgcn_raw_buffer_store_b64(wv, dvs, row_off + ct * 32 + g * 8, 0, kStoreAux);
-            } else {
-                __builtin_amdgcn_raw_buffer_store_b64(wk, dks, row_off + ct * 32 + g * 8, 0, 0);
-                __builtin_amdgcn_raw_buffer_store_b64(wv, dvs, row_off + ct * 32 + g * 8, 0, 0);
-            }
+            kw[ct] = pack_acc<DT>(acck[ct], scale);
+            vw[ct] = pack_acc<DT>(accv[ct], 1.f);
         }
+        store_tile<C>(dks, row_off, kw, g, whole_lines);
+        store_tile<C>(dvs, row_off, vw, g, whole_lines);
     }
 
     if (drpb && tid < W) {              // rsum was complete at the barriers before pass 2

@@ -263,6 +263,38 @@ __device__ inline float xor_sum(float x) {
     return a + b;
 }
 
+// ---- tile stores -------------------------------------------------------------------
+// Pack an accumulator (lane (n, g): row n, channels 16*ct + 4g .. 4g+3) times `f` into four 16-bit values.
+template <class DT> __device__ inline u32x2 pack_acc(f32x4 a, float f) {
+    return u32x2{Mma<DT>::pack(a[0] * f, a[1] * f), Mma<DT>::pack(a[2] * f, a[3] * f)};
+}
+// Store a 16 x C tile held as one u32x2 per channel tile.  Channel tiles are paired so that a lane writes 16
+// contiguous bytes: v_permlane16_swap hands lanes of even g the neighbour's half of the even tile and lanes of odd
+// g the neighbour's half of the odd tile.  Half as many stores, and one instruction writes whole 64-byte pieces of
+// a row instead of 32-byte halves that the other instruction completes later.
+template <int C, int AUX>
+__device__ inline void store_tile(Rsrc dst, int row_byte, const u32x2 (&w)[C / 16], int g) {
+    constexpr int CT = C / 16;
+    if constexpr (CT == 1) {
+        __builtin_amdgcn_raw_buffer_store_b64(w[0], dst, row_byte + g * 8, 0, AUX);
+    } else {
+#pragma unroll
+        for (int p = 0; p < CT / 2; ++p) {
+            const u32x2 lo = __builtin_amdgcn_permlane16_swap(w[2 * p].x, w[2 * p + 1].x, false, false);
+            const u32x2 hi = __builtin_amdgcn_permlane16_swap(w[2 * p].y, w[2 * p + 1].y, false, false);
+            const u32x4 v = {lo.x, hi.x, lo.y, hi.y};
+            __builtin_amdgcn_raw_buffer_store_b128(v, dst, row_byte + (2 * p + (g & 1)) * 32 + (g >> 1) * 16, 0, AUX);
+        }
+    }
+}
+template <int C>
+__device__ inline void store_tile(Rsrc dst, int row_byte, const u32x2 (&w)[C / 16], int g, bool stream) {
+    if (stream)
+        store_tile<C, kStoreAux>(dst, row_byte, w, g);
+    else
+        store_tile<C, 0>(dst, row_byte, w, g);
+}
+
 // ---- window slots of a lane ------------------------------------------------------
 template <int NBV> struct Window {
     // slot sets: X = block 0 (NBV 2) or merged blocks 0/2 (NBV 3);  Y = block 1

@@ -162,13 +162,10 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
             for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr(blk + v_lane.off[ct]), pb, o[ct]);
         }
         const int qrow = 16 * i + n;
+        u32x2 ow[CT];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            u32x2 w;
-            w.x = Mma<DT>::pack(o[ct][0], o[ct][1]);
-            w.y = Mma<DT>::pack(o[ct][2], o[ct][3]);
-            __builtin_amdgcn_raw_buffer_store_b64(w, os, qrow * (2 * C) + ct * 32 + g * 8, 0, kStoreAux);
-        }
+        for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], 1.f);
+        store_tile<C, kStoreAux>(os, qrow * (2 * C), ow, g);
     }
 }
 
@@ -231,13 +228,10 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
             for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(xt + x_tr.off[ct]), pb, acc[ct]);
         }
         const int row_off = (16 * (kp - i0) - shift + n) * (2 * C);     // outside the strip -> dropped
+        u32x2 ow[CT];
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            u32x2 w;
-            w.x = Mma<DT>::pack(acc[ct][0], acc[ct][1]);
-            w.y = Mma<DT>::pack(acc[ct][2], acc[ct][3]);
-            __builtin_amdgcn_raw_buffer_store_b64(w, os, row_off + ct * 32 + g * 8, 0, kStoreAux);
-        }
+        for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(acc[ct], 1.f);
+        store_tile<C>(os, row_off, ow, g, stores_whole_lines(2 * C, C, shift));
     }
 }
 
