@@ -13,12 +13,13 @@ __global__ void __launch_bounds__(kThreads)
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
-                 int strips, float scale, uint32_t strips_magic, uint32_t heads_magic, Strides in, Strides outl) {
+                 int strips, float scale, uint32_t strips_magic, uint32_t heads_magic, Strides in, Strides outl,
+                 int shift) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = Strip<C>::kMaxTiles;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
-                   in.sample, in.head, in.pitch, outl.sample, outl.head, outl.pitch);
+                   in.sample, in.head, in.pitch, outl.sample, outl.head, outl.pitch, shift);
     // dynamic LDS (launch_fwd): K and V regions of nt+2 tiles starting one tile before the strip (row 16*i0 - 16:
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
     // forward is not short of LDS), Q region of nt tiles
@@ -34,7 +35,6 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     const uint32_t b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
     const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
-    const int shift = NBV == 3 ? 16 : L;
 
     // resources end with the strip (plus its halo), so the fixed-size copy below
     // fetches nothing beyond what this strip needs
@@ -172,7 +172,7 @@ int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                                                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
                                                  sp.nt, sp.strips, scale, div_magic(sp.strips), div_magic(g.H),
-                                                 byte_strides(in), byte_strides(outl));
+                                                 byte_strides(in), byte_strides(outl), window_shift(g));
     return launch_status();
 }
 
@@ -236,13 +236,13 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes, uint32_t strips_magic,
-                 uint32_t heads_magic, Strides in, Strides outl) {
+                 uint32_t heads_magic, Strides in, Strides outl, int shift) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
                    drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, outl.sample,
-                   outl.head, outl.pitch);
+                   outl.head, outl.pitch, shift);
     constexpr int kRowsQ = (MT + 2) * 16;
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
@@ -267,7 +267,6 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     const uint32_t item = wi.item, b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
     const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
-    const int shift = NBV == 3 ? 16 : L;
 
     const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
     {
@@ -531,7 +530,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                                                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
                                                  t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
                                                  sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
-                                                 div_magic(g.H), byte_strides(in), byte_strides(outl));
+                                                 div_magic(g.H), byte_strides(in), byte_strides(outl), window_shift(g));
     if (partial && drpb)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();

@@ -428,6 +428,16 @@ inline int window_blocks(const Geom &g) {
     return 0;
 }
 
+// Rows between the first virtual key block and its query tile.  Three blocks: 16.  Two blocks: anything in
+// [L, 16 - R] covers the window; the first multiple of a 128-byte line's worth of rows is taken, so that key
+// blocks (the units dK / dV are written in) and the key-side copies start on a line.
+inline int window_shift(const Geom &g) {
+    if (window_blocks(g) != 2) return 16;
+    const int R = g.W - 1 - g.L, rows = std::max(1, 128 / (2 * g.C));
+    const int s = (g.L + rows - 1) / rows * rows;
+    return s <= 16 - R ? s : g.L;
+}
+
 #define NA1D_MFMA_DISPATCH(FN, ...)                                            \
     do {                                                                       \
         if (dtype == NA1D_BF16) {                                              \
