@@ -350,6 +350,32 @@ def test_model_shape_properties_at_full_size(dtype):
     assert (ones.float() - 1).abs().max().item() < (2e-2 if dtype == torch.bfloat16 else 4e-3)
 
 
+def test_tensors_beyond_4_gib_are_addressed_with_64_bit_offsets():
+    """B*T*C*2 bytes > 2^32 per tensor: the first and the last sequences of the big call must equal the same
+    sequences run alone, bit for bit (the reference indexes with 32-bit ints and cannot run this size)."""
+    B, T, C, W, L = 2200, 8000, 128, 15, 7
+    assert B * T * C * 2 > 2 ** 32
+    g = torch.Generator(device="cuda").manual_seed(1)
+    q, k, v, do = (torch.randn(B, T, C, device="cuda", dtype=torch.bfloat16, generator=g) for _ in range(4))
+    q.mul_(C ** -0.5)
+    out, lse = na1d_fused_forward_lse(q, k, v, W, L)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _lib.call_fused_backward(dq, dk, dv, None, q, k, v, out, do, lse, None, None, B, 1, T, C, W, L, 1.0)
+    for b in (0, B - 1):
+        sl = slice(b, b + 1)
+        o1, l1 = na1d_fused_forward_lse(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), W, L)
+        assert torch.equal(o1, out[sl]) and torch.equal(l1, lse[sl])
+        g1 = [torch.empty_like(o1) for _ in range(3)]
+        _lib.call_fused_backward(*g1, None, q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), o1,
+                                 do[sl].contiguous(), l1, None, None, 1, 1, T, C, W, L, 1.0)
+        for got, big in zip(g1, (dq, dk, dv)):
+            assert torch.equal(got, big[sl])
+    attn = torch.empty(B, T, W, device="cuda")
+    _unfused("na1d_qk_forward", attn, q, k, W, L)
+    a1 = _unfused("na1d_qk_forward", torch.empty(1, T, W, device="cuda"), q[B - 1:].contiguous(), k[B - 1:].contiguous(), W, L)
+    assert torch.equal(a1, attn[B - 1:])
+
+
 def test_deterministic_rpb_gradient_is_bit_reproducible():
     """With deterministic=True d rpb is folded in a fixed order: two runs give the same bits, and the
     atomics path agrees with it to fp32 rounding."""
