@@ -426,6 +426,47 @@ def test_two_kernel_families_agree(dtype):
     assert not torch.equal(fast[1], slow[1]) or not torch.equal(fast[3], slow[3])     # they really are different code
 
 
+def test_forward_and_backward_replay_from_a_hip_graph():
+    """The C ABI allocates nothing and launches only on the stream it is given, so a step can be captured once and
+    replayed: three replays on changing inputs, eager work in between, each checked against the eager result."""
+    N, H, T, C, W, L = 4, 4, 150, 16, 27, 13
+    B = N * H
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    new = lambda *shape: torch.randn(*shape, device="cuda", generator=gen)
+    q, k, v, do = (new(B, T, C).to(torch.bfloat16) for _ in range(4))
+    rpb = new(H, W) * 0.3
+    tv = torch.tensor([T, T - 9, 70, 1], dtype=torch.int32, device="cuda")
+    out, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    lse = torch.empty(B, T, device="cuda")
+    drpb = torch.zeros(H, W, device="cuda")
+    nbytes = _lib.fused_backward_workspace_bytes(B, H, T, C, W, L, q.dtype)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+
+    def step():
+        drpb.zero_()                                   # a fill kernel, not a memset node
+        _lib.call_fused_forward(out, lse, q, k, v, rpb, tv, B, H, T, C, W, L, 1.0)
+        _lib.call_fused_backward(dq, dk, dv, drpb, q, k, v, out, do, lse, rpb, tv, B, H, T, C, W, L, 1.0, workspace=ws)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                                         # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for t in (q, k, v, do):
+            t.copy_(new(B, T, C).to(torch.bfloat16))   # eager work between the replays
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in (out, lse, dq, dk, dv, drpb)]
+        step()
+        torch.cuda.synchronize()
+        for a, b in zip(got, (out, lse, dq, dk, dv, drpb)):
+            assert torch.equal(a, b), rep              # the workspace path makes d rpb reproducible too
+
+
 def test_runs_on_the_current_stream():
     """Launches go to torch's current stream (the reference uses the legacy default
     stream; its data prefetcher runs a side stream, public/Utils.py:89-100)."""
