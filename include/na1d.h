@@ -165,6 +165,17 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb,
                                 const int64_t *qkv_strides, const int64_t *out_strides,
                                 void *workspace, int64_t workspace_bytes, void *stream);
 
+/*
+ * Profiling hook; no counterpart in the reference.  From this call on, the matrix-core fused kernels that the
+ * CALLING THREAD launches record `start` just before and `stop` just after the kernel itself (hipEvent_t handles,
+ * recorded by hipExtLaunchKernel: the dispatch's own begin and end, i.e. what a profiler's kernel trace reports,
+ * without the gaps between launches that events recorded on the stream include).  Each launch re-records the same
+ * pair, so read them (hipEventElapsedTime) or change them between launches.  NULL, NULL switches it off.  With the
+ * workspace path of the backward the pair brackets the main kernel, not the small reduction that follows.  Not for
+ * use under stream capture.
+ */
+int na1d_profile_events(void *start, void *stop);
+
 /* Bytes of workspace na1d_fused_backward can use for these arguments (0 if it has
  * no use for one, negative status on invalid arguments). */
 int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,

@@ -4,6 +4,13 @@
 
 #include "na1d_common.h"
 
+namespace na1d {
+LaunchEvents &launch_events() {
+    static thread_local LaunchEvents events;
+    return events;
+}
+}  // namespace na1d
+
 namespace {
 
 using na1d::Geom;
@@ -201,6 +208,13 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb, const
     if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;
     return na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, nullptr, dout, lse, rpb, t_valid, g, in, outl, scale, dtype,
                                  (float *)workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
+}
+
+int na1d_profile_events(void *start, void *stop) {
+    na1d::LaunchEvents &ev = na1d::launch_events();
+    ev.start = (hipEvent_t)start;
+    ev.stop = (hipEvent_t)stop;
+    return NA1D_OK;
 }
 
 int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,

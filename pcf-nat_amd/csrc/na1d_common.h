@@ -80,6 +80,14 @@ struct Layout {
 };
 inline Layout packed_layout(const Geom &g) { return Layout{(int64_t)g.H * g.T * g.C, g.T * g.C, g.C}; }
 
+// Optional pair of events that the fused launches of the calling thread record tightly around the kernel
+// (hipExtLaunchKernel: the dispatch's own start and end, what a profiler's kernel trace reports) - see
+// na1d_profile_events() in na1d.h.  Null, the default, means ordinary launches.
+struct LaunchEvents {
+    hipEvent_t start = nullptr, stop = nullptr;
+};
+LaunchEvents &launch_events();   // thread-local, lives in na1d_api.cpp
+
 // Host-side launch status check.
 inline int launch_status() { return hipGetLastError() == hipSuccess ? NA1D_OK : NA1D_ERR_LAUNCH; }
 

@@ -169,10 +169,9 @@ int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *
     auto kern = window_blocks(g) == 2 ? fused_fwd_kernel<DT, C, 2> : fused_fwd_kernel<DT, C, 3>;
     const size_t lds = (size_t)2 * region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
-                                                 rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
-                                                 sp.nt, sp.strips, scale, div_magic(sp.strips), div_magic(g.H),
-                                                 byte_strides(in), byte_strides(outl), window_shift(g));
+    launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
+                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
+                  div_magic(sp.strips), div_magic(g.H), byte_strides(in), byte_strides(outl), window_shift(g));
     return launch_status();
 }
 
@@ -526,11 +525,10 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
                        (kThreads + (drpb ? kWaves * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
-                                                 (const char *)k, (const char *)v, (const char *)dout, lse, rpb,
-                                                 t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles,
-                                                 sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
-                                                 div_magic(g.H), byte_strides(in), byte_strides(outl), window_shift(g));
+    launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
+                  (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
+                  g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
+                  div_magic(g.H), byte_strides(in), byte_strides(outl), window_shift(g));
     if (partial && drpb)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();

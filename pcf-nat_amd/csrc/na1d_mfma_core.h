@@ -38,6 +38,8 @@
 
 #include <algorithm>
 
+#include <hip/hip_ext.h>
+
 #include "na1d_common.h"
 
 namespace na1d {
@@ -408,6 +410,16 @@ __device__ inline uint32_t xcd_item(uint32_t wg, uint32_t items) {
     const uint32_t per = items / 8;          // items in the evenly dealt part
     if (wg >= per * 8) return wg;            // ragged tail keeps its id
     return (wg & 7) * per + (wg >> 3);
+}
+
+// Launch, with the calling thread's profiling events around the kernel if it has set any.
+template <class K, class... Args>
+inline void launch_kernel(K kern, unsigned grid, size_t lds, hipStream_t s, Args... args) {
+    const LaunchEvents &ev = launch_events();
+    if (ev.start || ev.stop)
+        hipExtLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), (uint32_t)lds, s, ev.start, ev.stop, 0, args...);
+    else
+        kern<<<grid, kThreads, lds, s>>>(args...);
 }
 
 // Dynamic LDS above 64 KB has to be allowed per kernel.

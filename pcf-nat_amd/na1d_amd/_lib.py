@@ -21,7 +21,7 @@ _i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_
 _UNFUSED = ("na1d_qk_forward", "na1d_av_forward", "na1d_q_backward", "na1d_k_backward",
             "na1d_a_backward", "na1d_v_backward")
 SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_backward_workspace_bytes",
-                      "na1d_fused_forward_strided", "na1d_fused_backward_strided",
+                      "na1d_fused_forward_strided", "na1d_fused_backward_strided", "na1d_profile_events",
                       "na1d_version", "na1d_status_string")
 UNSUPPORTED = -8
 
@@ -60,6 +60,8 @@ def load():
     lib.na1d_fused_backward_strided.argtypes = [_ptr] * 11 + [_i64] * 6 + [_f32, _int, _ptr, _ptr, _ptr, _i64, _ptr]
     lib.na1d_fused_backward_workspace_bytes.restype = _i64
     lib.na1d_fused_backward_workspace_bytes.argtypes = [_i64] * 6 + [_int]
+    lib.na1d_profile_events.restype = _int
+    lib.na1d_profile_events.argtypes = [_ptr, _ptr]
     lib.na1d_version.restype = _int
     lib.na1d_version.argtypes = []
     lib.na1d_status_string.restype = ctypes.c_char_p
