@@ -467,6 +467,32 @@ def test_forward_and_backward_replay_from_a_hip_graph():
             assert torch.equal(a, b), rep              # the workspace path makes d rpb reproducible too
 
 
+def test_profile_events_bracket_the_kernel():
+    """na1d_profile_events: the pair is recorded around the kernel by the launch itself; switched off again, launches
+    are ordinary ones."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    lib = _lib.load()
+    a, b = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
+    q, k, v = dev(*make_inputs(512, 300, 32, 15, 2, torch.float16, n=3))
+    want, _ = na1d_fused_forward_lse(q, k, v, 15, 7)
+    assert lib.na1d_profile_events(a, b) == 0
+    try:
+        got, _ = na1d_fused_forward_lse(q, k, v, 15, 7)
+    finally:
+        assert lib.na1d_profile_events(None, None) == 0
+    torch.cuda.synchronize()
+    ms = ctypes.c_float()
+    assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+    assert 1e-3 < ms.value < 1.0                      # a few microseconds of kernel, not a stream's worth of gaps
+    assert torch.equal(got, want)
+    again, _ = na1d_fused_forward_lse(q, k, v, 15, 7)
+    assert torch.equal(again, want)
+    hip.hipEventDestroy(a)
+    hip.hipEventDestroy(b)
+
+
 def test_runs_on_the_current_stream():
     """Launches go to torch's current stream (the reference uses the legacy default
     stream; its data prefetcher runs a side stream, public/Utils.py:89-100)."""
