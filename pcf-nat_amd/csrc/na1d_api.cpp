@@ -72,6 +72,15 @@ inline bool mfma_allowed() {
     return !(e && e[0] == '1');
 }
 
+// The matrix-core forward: the two/three-block kernel where it covers the window, else the wide-window one.
+int mfma_fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+                   const int32_t *t_valid, const Geom &g, const na1d::Layout &in, const na1d::Layout &outl, float scale,
+                   int dtype, hipStream_t s) {
+    const int st = na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, dtype, s);
+    if (st != NA1D_ERR_UNSUPPORTED) return st;
+    return na1d::mfma::wide_fwd(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, dtype, s);
+}
+
 int band_qk(void *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s) {
     const int st = mfma_allowed() ? na1d::mfma::qk((float *)attn, a, b, g, dtype, s) : NA1D_ERR_UNSUPPORTED;
     return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::qk((float *)attn, a, b, g, dtype, s) : st;
@@ -149,8 +158,8 @@ int na1d_fused_forward(void *out, float *lse, const void *q, const void *k, cons
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
     const na1d::Layout packed = na1d::packed_layout(g);
-    const int st = mfma_allowed() ? na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, packed, packed, scale,
-                                                          dtype, (hipStream_t)stream)
+    const int st = mfma_allowed() ? mfma_fused_fwd(out, lse, q, k, v, rpb, t_valid, g, packed, packed, scale, dtype,
+                                                   (hipStream_t)stream)
                                   : NA1D_ERR_UNSUPPORTED;
     if (st != NA1D_ERR_UNSUPPORTED) return st;
     return na1d::generic::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream);
@@ -188,7 +197,7 @@ int na1d_fused_forward_strided(void *out, float *lse, const void *q, const void 
     const int ls = check_layout(qkv_strides, g, in), lo = check_layout(out_strides, g, outl);
     if (ls != NA1D_OK || lo != NA1D_OK) return ls != NA1D_OK ? ls : lo;
     if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;
-    return na1d::mfma::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, dtype, (hipStream_t)stream);
+    return mfma_fused_fwd(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, dtype, (hipStream_t)stream);
 }
 
 int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k,

@@ -270,6 +270,44 @@ def test_strided_entry_points_leave_the_gaps_alone(dtype):
     assert not torch.isnan(gbuf[..., :C]).any()
 
 
+WIDE_GEOMS = [  # (N, H, T, C, W, left): windows the two/three-block kernels do not cover
+    (2, 2, 100, 16, 33, 16), (2, 2, 130, 32, 40, 7), (1, 2, 90, 64, 48, 47), (2, 1, 200, 16, 64, 0), (1, 2, 70, 128, 65, 32),
+    (2, 2, 300, 32, 80, 39), (1, 3, 45, 16, 80, 79), (2, 2, 17, 32, 80, 0), (1, 1, 500, 64, 27, 20), (2, 2, 64, 16, 31, 30),
+    (1, 2, 1, 16, 80, 40), (2, 4, 257, 32, 49, 24),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", WIDE_GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_wide_windows_match_oracle(geom, dtype):
+    """W up to 80 and lopsided windows (more than 16 keys on one side) on the matrix-core path."""
+    N, H, T, C, W, L = geom
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, W, 77, dtype, n=4, scale=C ** -0.5)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(9)) * 0.5
+    pad = torch.tensor([0, T // 2, T][:N] + [1] * max(0, N - 3))
+    t_valid = (T - pad).to(torch.int32).cuda()
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    rd = rpb.cuda().requires_grad_(True)
+    out = na1d_fused(qd, kd, vd, W, L, rpb=rd, t_valid=t_valid, num_heads=H)
+    out.backward(do.cuda())
+    want_o, _, want_lse = O.na1d_forward(q.float(), k.float(), v.float(), W, L, rpb, pad, H)
+    wq, wk, wv, wr = O.na1d_backward(q.float(), k.float(), v.float(), do.float(), W, L, rpb, pad, H)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float(), want_o) < tol, "O"
+    _, lse = na1d_fused_forward_lse(qd.detach(), kd.detach(), vd.detach(), W, L, rd.detach(), t_valid, H)
+    assert torch.allclose(lse.cpu(), want_lse, atol=2e-3, rtol=1e-4), "LSE"
+    for name, got, want in (("dQ", qd.grad, wq), ("dK", kd.grad, wk), ("dV", vd.grad, wv)):
+        assert O.rel_l2(got.float(), want) < tol, name
+    assert _err(rd.grad, wr) < tol, "drpb"
+    os.environ["NA1D_FORCE_GENERIC"] = "1"          # the generic kernels are the second opinion
+    try:
+        ref, _ = na1d_fused_forward_lse(qd.detach(), kd.detach(), vd.detach(), W, L, rd.detach(), t_valid, H)
+    finally:
+        del os.environ["NA1D_FORCE_GENERIC"]
+    assert O.rel_l2(out.float(), ref.float()) < tol
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
 def test_fused_scale_argument_and_optional_inputs(dtype):
     """scale multiplies the fp32 scores; rpb / t_valid / lse are optional."""
