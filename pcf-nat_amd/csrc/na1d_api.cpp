@@ -81,6 +81,16 @@ int mfma_fused_fwd(void *out, float *lse, const void *q, const void *k, const vo
     return na1d::mfma::wide_fwd(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, dtype, s);
 }
 
+int mfma_fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+                   const void *out, const void *dout, const float *lse, const float *rpb, const int32_t *t_valid,
+                   const Geom &g, const na1d::Layout &in, const na1d::Layout &outl, float scale, int dtype,
+                   float *workspace, int64_t workspace_bytes, hipStream_t s) {
+    const int st = na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, in, outl, scale,
+                                         dtype, workspace, workspace_bytes, s);
+    if (st != NA1D_ERR_UNSUPPORTED) return st;
+    return na1d::mfma::wide_bwd(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, dtype, s);
+}
+
 int band_qk(void *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s) {
     const int st = mfma_allowed() ? na1d::mfma::qk((float *)attn, a, b, g, dtype, s) : NA1D_ERR_UNSUPPORTED;
     return st == NA1D_ERR_UNSUPPORTED ? na1d::generic::qk((float *)attn, a, b, g, dtype, s) : st;
@@ -176,8 +186,8 @@ int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb, const void *q
         return NA1D_ERR_ALIGN;
     if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
     const na1d::Layout packed = na1d::packed_layout(g);
-    const int st = mfma_allowed() ? na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g,
-                                                          packed, packed, scale, dtype, (float *)workspace,
+    const int st = mfma_allowed() ? mfma_fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g,
+                                                   packed, packed, scale, dtype, (float *)workspace,
                                                           workspace ? workspace_bytes : 0, (hipStream_t)stream)
                                   : NA1D_ERR_UNSUPPORTED;
     if (st != NA1D_ERR_UNSUPPORTED) return st;
@@ -215,8 +225,8 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb, const
     const int ls = check_layout(qkv_strides, g, in), lo = check_layout(out_strides, g, outl);
     if (ls != NA1D_OK || lo != NA1D_OK) return ls != NA1D_OK ? ls : lo;
     if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;
-    return na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, nullptr, dout, lse, rpb, t_valid, g, in, outl, scale, dtype,
-                                 (float *)workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
+    return mfma_fused_bwd(dq, dk, dv, drpb, q, k, v, nullptr, dout, lse, rpb, t_valid, g, in, outl, scale, dtype,
+                          (float *)workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
 }
 
 int na1d_profile_events(void *start, void *stop) {

@@ -123,6 +123,9 @@ int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype);   // 0 when the sha
 int wide_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
              const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &out_layout, float scale,
              int dtype, hipStream_t s);
+int wide_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v, const void *dout,
+             const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g, const Layout &in,
+             const Layout &out_layout, float scale, int dtype, hipStream_t s);
 }  // namespace mfma
 
 }  // namespace na1d
