@@ -7,19 +7,39 @@
 //
 // P2 and P3 round the scores to the 16-bit dtype before the contraction, as the
 // reference kernels do (bf16_ana1d_kernel.cu:305,414); accumulation is fp32.
+//
+// A query tile meets NBV = 2 .. 6 virtual key blocks (W up to 80); the first one starts `shift` rows before
+// the tile, shift in [L, 16*NBV - 16 - R], on a 128-byte line where that is possible.
 #include "na1d_mfma_core.h"
 
 namespace na1d {
 namespace mfma {
+
+struct BandCover {
+    int nbv, shift, max_tiles;   // 0 blocks: shape not covered
+};
+inline BandCover band_cover(const Geom &g) {
+    BandCover c{0, 0, 0};
+    if (g.C != 16 && g.C != 32 && g.C != 64 && g.C != 128) return c;
+    if (g.T > (1 << 29) / g.C || g.T > (1 << 29) / (4 * g.W) || g.W > NA1D_MAX_WINDOW) return c;
+    c.nbv = std::max(2, (15 + g.W + 15) / 16);
+    const int R = g.W - 1 - g.L, rows = std::max(1, 128 / (2 * g.C));
+    const int hi = 16 * c.nbv - 16 - R, s16 = (g.L + 15) / 16 * 16, s = (g.L + rows - 1) / rows * rows;
+    c.shift = s16 <= hi ? s16 : s <= hi ? s : g.L;      // whole tiles, else whole lines, else the first key
+    c.max_tiles = c.nbv <= 3 ? (g.C <= 32 ? 8 : g.C <= 64 ? 4 : 2) : (g.C <= 64 ? 4 : 2);
+    return c;
+}
+constexpr int kBandMaxTiles = 8;          // compile-time ceiling of max_tiles
 
 // Copy `floats` fp32 values starting `first` floats into a sequence's score rows straight into LDS, one
 // 1 KB chunk per wave and round (see stage_direct); the buffer resource zero-fills what lies outside the
 // rows the strip needs.  `first` is a tile start, so 16-byte units never straddle the sequence's start.
 // The region is padded to whole chunks (score_bytes).
 inline __host__ __device__ int score_bytes(int tiles, int W) { return (tiles * 16 * W * 4 + kChunk - 1) / kChunk * kChunk; }
-template <int C>
+template <int NBV>
 __device__ inline void stage_scores(Rsrc src, int first, LDS_PTR(float) region, int tiles, int W, int wave, int lane) {
-    constexpr int kRounds = ((Strip<C>::kMaxTiles + 2) * 16 * 32 * 4 / kChunk + kWaves - 1) / kWaves;   // W <= 32
+    // at most kBandMaxTiles + NBV tiles of 16 rows of W <= 16*NBV - 15 floats
+    constexpr int kRounds = (((kBandMaxTiles + NBV) * 16 * (16 * NBV - 15) * 4 + kChunk - 1) / kChunk + kWaves - 1) / kWaves;
     const int chunks = score_bytes(tiles, W) / kChunk;
 #pragma unroll
     for (int j = 0; j < kRounds; ++j) {
@@ -41,14 +61,16 @@ __device__ inline float score_at(LDS_PTR(float) rows, int row, int j, int W) {  
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__restrict__ kb, uint32_t items, int T,
-          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic) {
+          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift) {
     using LL = Lds<C>;
-    constexpr int MT = Strip<C>::kMaxTiles;
-    fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic);
-    // dynamic LDS: K region of nt+2 tiles, Q region of nt tiles, one 16 x W fp32 tile per wave
+    constexpr int MT = kBandMaxTiles;
+    fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic, shift);
+    // dynamic LDS: K region of kt tiles starting sb tiles before the strip, Q region of nt tiles, one 16 x W fp32
+    // tile per wave
+    const int sb = (shift + 15) >> 4, kt = nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) q_lds = k_lds + region_bytes<C>(nt + 2);
+    LDS_PTR(char) q_lds = k_lds + region_bytes<C>(kt);
     LDS_PTR(float) out_lds = (LDS_PTR(float))(q_lds + region_bytes<C>(nt));
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -58,18 +80,17 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     const int strip = (int)(item - b * strips);
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
-    const int shift = NBV == 3 ? 16 : L;
 
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
-        const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
+        const int key_bytes = min(T, 16 * (i0 - sb + kt)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
         const int lane_off = direct_lane_offset<C>(wave, lane);
-        stage_direct<C, MT + 2, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * i0 - 16, k_lds, nt + 2, wave, lane_off);
+        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off);
         stage_direct<C, MT, kReadShared>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off);
     }
     const Rsrc as = make_rsrc(attn + (int64_t)b * T * W, T * W * 4);
     RowLane<C> k_lane, q_lane;
-    k_lane.init(16 - shift, lane);
+    k_lane.init(16 * sb - shift, lane);
     q_lane.init(0, lane);
     LDS_PTR(float) mine = out_lds + wave * 16 * W;
     wait_direct();
@@ -113,15 +134,16 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ v, uint32_t items, int T,
-          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic) {
+          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
-    constexpr int MT = Strip<C>::kMaxTiles;
-    fetch_args_now(out, attn, v, items, T, W, L, tiles, nt, strips, strips_magic);
-    // dynamic LDS: V region of nt+2 tiles, score rows of the strip (nt*16 x W fp32)
+    constexpr int MT = kBandMaxTiles;
+    fetch_args_now(out, attn, v, items, T, W, L, tiles, nt, strips, strips_magic, shift);
+    // dynamic LDS: V region of kt tiles starting sb tiles before the strip, score rows of the strip (nt*16 x W fp32)
+    const int sb = (shift + 15) >> 4, kt = nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) v_lds = (LDS_PTR(char))smem;
-    LDS_PTR(float) s_lds = (LDS_PTR(float))(v_lds + region_bytes<C>(nt + 2));
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(v_lds + region_bytes<C>(kt));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -130,18 +152,17 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
     const int strip = (int)(item - b * strips);
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
-    const int shift = NBV == 3 ? 16 : L;
 
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
-        const int key_bytes = min(T, 16 * (i1 + 1)) * 2 * C;
-        stage_direct<C, MT + 2, kReadShared>(make_rsrc(v + seq_off, key_bytes), 16 * i0 - 16, v_lds, nt + 2, wave,
-                                direct_lane_offset<C>(wave, lane));
-        stage_scores<C>(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, s_lds, nt, W, wave, lane);
+        const int key_bytes = min(T, 16 * (i0 - sb + kt)) * 2 * C;
+        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(v + seq_off, key_bytes), 16 * (i0 - sb), v_lds, kt, wave,
+                                               direct_lane_offset<C>(wave, lane));
+        stage_scores<NBV>(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, s_lds, nt, W, wave, lane);
     }
     const Rsrc os = make_rsrc(out + seq_off, T * 2 * C);
     TrLane<C> v_lane;
-    v_lane.init(16 - shift, lane);
+    v_lane.init(16 * sb - shift, lane);
     wait_direct();
     __syncthreads();
 
@@ -175,15 +196,18 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ x, uint32_t items,
-              int T, int W, int L, int tiles, int nt, int strips, uint32_t strips_magic) {
+              int T, int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
-    constexpr int MT = Strip<C>::kMaxTiles;
-    fetch_args_now(out, attn, x, items, T, W, L, tiles, nt, strips, strips_magic);
-    // dynamic LDS: x rows of query tiles i0-1 .. i1 (nt+2 tiles) and their score rows ((nt+2)*16 x W fp32)
+    constexpr int MT = kBandMaxTiles;
+    fetch_args_now(out, attn, x, items, T, W, L, tiles, nt, strips, strips_magic, shift);
+    // Key block kp (rows 16*kp - shift ...) is virtual block vb of query tile kp - vb, so the blocks that touch the
+    // strip's rows need the query tiles i0 - hb .. i1 - 1 + ha.  Dynamic LDS: their x rows (qtiles tiles) and their
+    // score rows (qtiles*16 x W fp32)
+    const int hb = NBV - 1 - (shift >> 4), ha = (shift + 15) >> 4, qtiles = nt + hb + ha;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) x_lds = (LDS_PTR(char))smem;
-    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + region_bytes<C>(nt + 2));
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + region_bytes<C>(qtiles));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -192,14 +216,14 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     const int strip = (int)(item - b * strips);
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
-    const int shift = NBV == 3 ? 16 : L;
+    const int q0 = i0 - hb;                                            // first query tile needed
 
     const int64_t seq_off = (int64_t)b * T * (2 * C);
     {
-        const int rows_hi = min(T, 16 * (i1 + 1));
-        stage_direct<C, MT + 2, kReadShared>(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * i0 - 16, x_lds, nt + 2, wave,
-                                direct_lane_offset<C>(wave, lane));
-        stage_scores<C>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), (16 * i0 - 16) * W, s_lds, nt + 2, W, wave, lane);
+        const int rows_hi = min(T, 16 * (q0 + qtiles));
+        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * q0, x_lds, qtiles, wave,
+                                               direct_lane_offset<C>(wave, lane));
+        stage_scores<NBV>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), 16 * q0 * W, s_lds, qtiles, W, wave, lane);
     }
     TrLane<C> x_tr;
     x_tr.init(0, lane);
@@ -210,14 +234,14 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
 
     // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb; lane (n, g)
     // holds key row n of the block against queries 4g+r of that tile: slot j = 16*vb - shift + n - (4g+r) + L
-    const int kp_lo = i0 + (shift == 16 ? 1 : 0), kp_hi = i1 - (shift == 0 ? 1 : 0);
+    const int kp_lo = i0 + (shift >> 4), kp_hi = i1 - 1 + ha;
     for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
         f32x4 acc[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
-            const int tq = kp - vb - (i0 - 1);
+            const int tq = kp - vb - q0;                               // in [0, qtiles) by the choice of hb and ha
             LDS_PTR(float) rows = s_lds + tq * 16 * W;
             float p[4];
 #pragma unroll
@@ -236,55 +260,103 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
 }
 
 // ----------------------------------------------------------------------------- launchers
+constexpr size_t kLdsPerCu = 160 * 1024;
+
+// Strip length: the cover's ceiling, shortened until the workgroup's LDS (a function of it) fits a CU.
+template <class F>
+inline int fit_tiles(int max_tiles, F lds_of) {
+    int nt = max_tiles;
+    while (nt >= 1 && lds_of(nt) > kLdsPerCu) --nt;
+    return nt;
+}
+
+template <class DT, int C, int NBV>
+int launch_qk_n(float *attn, const void *a, const void *b, const Geom &g, const BandCover &c, hipStream_t s) {
+    auto lds_of = [&](int nt) {
+        return (size_t)region_bytes<C>(nt - 1 + NBV + ((c.shift & 15) ? 1 : 0)) + region_bytes<C>(nt) +
+               (size_t)kWaves * 16 * g.W * sizeof(float);
+    };
+    const int mt = fit_tiles(c.max_tiles, lds_of);
+    if (mt < 1) return NA1D_ERR_UNSUPPORTED;
+    const Split sp = make_split(g.B, g.T, mt);
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
+    auto kern = qk_kernel<DT, C, NBV>;
+    const size_t lds = lds_of(sp.nt);
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>(attn, (const char *)a, (const char *)b, (uint32_t)sp.items, (int)g.T,
+                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift);
+    return launch_status();
+}
+
+template <class DT, int C, int NBV>
+int launch_av_n(void *out, const float *attn, const void *v, const Geom &g, const BandCover &c, hipStream_t s) {
+    auto lds_of = [&](int nt) {
+        return (size_t)region_bytes<C>(nt - 1 + NBV + ((c.shift & 15) ? 1 : 0)) + score_bytes(nt, g.W);
+    };
+    const int mt = fit_tiles(c.max_tiles, lds_of);
+    if (mt < 1) return NA1D_ERR_UNSUPPORTED;
+    const Split sp = make_split(g.B, g.T, mt);
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
+    auto kern = av_kernel<DT, C, NBV>;
+    const size_t lds = lds_of(sp.nt);
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)v, (uint32_t)sp.items, (int)g.T, g.W,
+                                                   g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift);
+    return launch_status();
+}
+
+template <class DT, int C, int NBV>
+int launch_gather_n(void *out, const float *attn, const void *x, const Geom &g, const BandCover &c, hipStream_t s) {
+    const int halo = NBV - 1 - (c.shift >> 4) + ((c.shift + 15) >> 4);          // query tiles beyond the strip
+    auto lds_of = [&](int nt) { return (size_t)region_bytes<C>(nt + halo) + score_bytes(nt + halo, g.W); };
+    const int mt = fit_tiles(c.max_tiles, lds_of);
+    if (mt < 1) return NA1D_ERR_UNSUPPORTED;
+    const Split sp = make_split(g.B, g.T, mt);
+    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
+    auto kern = gather_kernel<DT, C, NBV>;
+    const size_t lds = lds_of(sp.nt);
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)x, (uint32_t)sp.items, (int)g.T, g.W,
+                                                   g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift);
+    return launch_status();
+}
+
+#define NA1D_BAND_BLOCKS(FN, ...)                          \
+    do {                                                   \
+        const BandCover c = band_cover(g);                 \
+        switch (c.nbv) {                                   \
+            case 2: return FN<DT, C, 2>(__VA_ARGS__, c, s); \
+            case 3: return FN<DT, C, 3>(__VA_ARGS__, c, s); \
+            case 4: return FN<DT, C, 4>(__VA_ARGS__, c, s); \
+            case 5: return FN<DT, C, 5>(__VA_ARGS__, c, s); \
+            case 6: return FN<DT, C, 6>(__VA_ARGS__, c, s); \
+        }                                                  \
+        return NA1D_ERR_UNSUPPORTED;                       \
+    } while (0)
+
 template <class DT, int C>
 int launch_qk(float *attn, const void *a, const void *b, const Geom &g, hipStream_t s) {
-    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
-    auto kern = window_blocks(g) == 2 ? qk_kernel<DT, C, 2> : qk_kernel<DT, C, 3>;
-    const size_t lds = (size_t)region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt) + (size_t)kWaves * 16 * g.W * sizeof(float);
-    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>(attn, (const char *)a, (const char *)b, (uint32_t)sp.items,
-                                                   (int)g.T, g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips));
-    return launch_status();
+    NA1D_BAND_BLOCKS(launch_qk_n, attn, a, b, g);
 }
-
 template <class DT, int C>
 int launch_av(void *out, const float *attn, const void *v, const Geom &g, hipStream_t s) {
-    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
-    auto kern = window_blocks(g) == 2 ? av_kernel<DT, C, 2> : av_kernel<DT, C, 3>;
-    const size_t lds = (size_t)region_bytes<C>(sp.nt + 2) + score_bytes(sp.nt, g.W);
-    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)v, (uint32_t)sp.items, (int)g.T,
-                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips));
-    return launch_status();
+    NA1D_BAND_BLOCKS(launch_av_n, out, attn, v, g);
 }
-
 template <class DT, int C>
 int launch_gather(void *out, const float *attn, const void *x, const Geom &g, hipStream_t s) {
-    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (sp.items > 0x7fffff00LL || !div_magic_ok(sp.items, sp.strips)) return NA1D_ERR_UNSUPPORTED;
-    auto kern = window_blocks(g) == 2 ? gather_kernel<DT, C, 2> : gather_kernel<DT, C, 3>;
-    const size_t lds = (size_t)region_bytes<C>(sp.nt + 2) + score_bytes(sp.nt + 2, g.W);
-    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)x, (uint32_t)sp.items, (int)g.T,
-                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips));
-    return launch_status();
+    NA1D_BAND_BLOCKS(launch_gather_n, out, attn, x, g);
 }
 
-// The score tensor is addressed with 32-bit byte offsets inside a sequence.
-inline bool scores_fit(const Geom &g) { return g.T <= (1 << 29) / (4 * g.W); }
-
 int qk(float *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s) {
-    if (!window_blocks(g) || !scores_fit(g)) return NA1D_ERR_UNSUPPORTED;
+    if (!band_cover(g).nbv) return NA1D_ERR_UNSUPPORTED;
     NA1D_MFMA_DISPATCH(launch_qk, attn, a, b, g, s);
 }
 int av(void *out, const float *attn, const void *v, const Geom &g, int dtype, hipStream_t s) {
-    if (!window_blocks(g) || !scores_fit(g)) return NA1D_ERR_UNSUPPORTED;
+    if (!band_cover(g).nbv) return NA1D_ERR_UNSUPPORTED;
     NA1D_MFMA_DISPATCH(launch_av, out, attn, v, g, s);
 }
 int gather(void *out, const float *attn, const void *x, const Geom &g, int dtype, hipStream_t s) {
-    if (!window_blocks(g) || !scores_fit(g)) return NA1D_ERR_UNSUPPORTED;
+    if (!band_cover(g).nbv) return NA1D_ERR_UNSUPPORTED;
     NA1D_MFMA_DISPATCH(launch_gather, out, attn, x, g, s);
 }
 

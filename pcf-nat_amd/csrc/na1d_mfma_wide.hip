@@ -23,8 +23,8 @@ inline WideCover wide_cover(const Geom &g) {
     if (c.nbv < 3) c.nbv = 3;
     // any shift in [L, 16*NBV - 16 - R] covers the window; prefer one that puts key blocks on 128-byte lines
     const int R = g.W - 1 - g.L, rows = std::max(1, 128 / (2 * g.C));
-    const int s = (g.L + rows - 1) / rows * rows;
-    c.shift = s <= 16 * c.nbv - 16 - R ? s : g.L;
+    const int hi = 16 * c.nbv - 16 - R, s16 = (g.L + 15) / 16 * 16, s = (g.L + rows - 1) / rows * rows;
+    c.shift = s16 <= hi ? s16 : s <= hi ? s : g.L;      // whole tiles, else whole lines, else the first key
     return c;
 }
 
