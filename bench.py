@@ -123,7 +123,7 @@ def oracle_attention(q, k, v, W, L, rpb=None, t_valid=None, num_heads=1):
 
 
 def model_inference(batch=256, frames=200, steps=10, warmup=3, cpu=True):
-    """PCF-NAT 4x4 inference (BASELINE config 3): bf16 autocast, random-init weights, 80-dim fbank-shaped
+    """PCF-NAT 4x4 inference (the reference's configs/pcf_nat4x4.yaml, batch 256 x 200 frames): bf16 autocast, random-init weights, 80-dim fbank-shaped
     N(0,1) input with the mean over time removed, fused NA1D in all 14 NA layers.  Returns embeddings/s on the
     GPU and, as a baseline, of the same model in PyTorch CPU fp32 on a bounded batch."""
     import torch
@@ -180,7 +180,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the op shards over "
-              "batch*heads with no exchange, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "batch*heads with no exchange between GPUs)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import torch

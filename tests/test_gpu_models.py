@@ -1,4 +1,5 @@
-"""BASELINE configs 3-5 at reduced batch: the GPU models (HIP operator, 16-bit autocast) against a CPU fp32
+"""The three model-level configurations (PCF-NAT 4x4 inference, PCF-NAT 6x4 variable length, MFA-NAT 4x4 training
+step) at reduced batch: the GPU models (HIP operator, 16-bit autocast) against a CPU fp32
 twin with the same state_dict whose attention is the oracle.  Bars: embedding cosine >= 0.999."""
 import pytest
 import torch
