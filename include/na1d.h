@@ -145,8 +145,8 @@ int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb,
  *   lse         : fp32 [N*H, T], packed
  * Strides must be multiples of 8 elements and row >= C; the caller guarantees that
  * distinct (n, h, t) rows do not overlap.  Returns NA1D_ERR_UNSUPPORTED when no
- * matrix-core kernel covers the shape (C not in {16, 32, 64, 128}): the caller then
- * packs the tensors and uses the packed entry points.  The backward needs no `out`.
+ * matrix-core kernel covers the shape (C > 128): the caller then packs the tensors
+ * and uses the packed entry points.  The backward needs no `out`.
  */
 int na1d_fused_forward_strided(void *out, float *lse,
                                const void *q, const void *k, const void *v,

@@ -19,7 +19,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = Strip<C>::kMaxTiles;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
-                   in.sample, in.head, in.pitch, outl.sample, outl.head, outl.pitch, shift);
+                   in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift);
     // dynamic LDS (launch_fwd): K and V regions of nt+2 tiles starting one tile before the strip (row 16*i0 - 16:
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
     // forward is not short of LDS), Q region of nt tiles
@@ -47,7 +47,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
 
     // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
     {
-        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch);
+        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
         if (strips == 1 && (in.pitch == 2 * C || C % 64 == 0)) {      // nobody else reads these rows' lines
             stage_direct<C, MT + 2, kReadOnce>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
             stage_direct<C, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
@@ -154,7 +154,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
-        store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines);
+        store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines, outl.width);
         if (g == 0)
             __builtin_amdgcn_raw_buffer_store_b32(
                 __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2), ls, qrow * 4, 0, 0);
@@ -171,7 +171,7 @@ int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
-                  div_magic(sp.strips), div_magic(g.H), byte_strides(in), byte_strides(outl), window_shift(g));
+                  div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g));
     return launch_status();
 }
 
@@ -240,8 +240,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
-                   drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, outl.sample,
-                   outl.head, outl.pitch, shift);
+                   drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width,
+                   outl.sample, outl.head, outl.pitch, outl.width, shift);
     constexpr int kRowsQ = (MT + 2) * 16;
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
@@ -274,8 +274,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         const Rsrc ks = make_rsrc(k + in_off, key_bytes), vs = make_rsrc(v + in_off, key_bytes);
         const Rsrc qs = make_rsrc(q + in_off, qry_rows * in.pitch), gs = make_rsrc(dout + out_off, qry_rows * outl.pitch);
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
-        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch);
-        const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch);
+        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
+        const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch, outl.width);
         // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * i0 - 16 + tid) * 4, 0, 0, 0);
         if (strips == 1 && (in.pitch == 2 * C || C % 64 == 0) && (outl.pitch == 2 * C || C % 64 == 0)) {
@@ -403,7 +403,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         u32x2 qw[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[ct], scale);
-        store_tile<C>(dqs, qrow * in.pitch, qw, g, dq_whole_lines);
+        store_tile<C>(dqs, qrow * in.pitch, qw, g, dq_whole_lines, in.width);
     }
 
     // d rpb: the window slot of each of a lane's 8 score registers is the same for every tile, so the lane
@@ -495,8 +495,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             kw[ct] = pack_acc<DT>(acck[ct], scale);
             vw[ct] = pack_acc<DT>(accv[ct], 1.f);
         }
-        store_tile<C>(dks, row_off, kw, g, whole_lines);
-        store_tile<C>(dvs, row_off, vw, g, whole_lines);
+        store_tile<C>(dks, row_off, kw, g, whole_lines, in.width);
+        store_tile<C>(dvs, row_off, vw, g, whole_lines, in.width);
     }
 
     if (drpb && tid < W) {              // rsum was complete at the barriers before pass 2
@@ -528,7 +528,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
-                  div_magic(g.H), byte_strides(in), byte_strides(outl), window_shift(g));
+                  div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g));
     if (partial && drpb)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();

@@ -155,12 +155,16 @@ static_assert(kWaves % 4 == 0, "chunk -> swizzle phase mapping assumes a multipl
 template <int C> constexpr int region_bytes(int ntiles) {
     return (ntiles * Lds<C>::kTileBytes + kChunk - 1) / kChunk * kChunk;
 }
-// `pitch` is the distance in bytes between consecutive rows in memory (2*C when the
-// rows are packed).
-template <int C> __device__ inline int direct_lane_offset(int wave, int lane, int pitch = Lds<C>::kRowBytes) {
+// `pitch` is the distance in bytes between consecutive rows in memory, `width` the bytes of a row that exist
+// there (2 * head_dim; both 2*C when the rows are packed and as wide as the kernel's C).  A head_dim below C is
+// zero-padded on the way in: the units past `width` ask for an address no resource reaches, and arrive as zeros.
+constexpr int kNowhere = 0x60000000;     // beyond any resource (they end below 2^30), whatever small offset is added
+template <int C>
+__device__ inline int direct_lane_offset(int wave, int lane, int pitch = Lds<C>::kRowBytes, int width = Lds<C>::kRowBytes) {
     const int u = wave * 64 + lane;      // 16-byte unit inside chunks wave, wave + 4, ...
     const int su = u % Lds<C>::kUnits;
-    return (lane / Lds<C>::kUnits) * pitch + (su ^ Lds<C>::swz(u / Lds<C>::kUnits)) * 16;
+    const int unit = su ^ Lds<C>::swz(u / Lds<C>::kUnits);
+    return unit * 16 < width ? (lane / Lds<C>::kUnits) * pitch + unit * 16 : kNowhere;
 }
 template <int C, int NTILES, int AUX>
 __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, int ntiles, int wave, int lane_off,
@@ -275,26 +279,27 @@ template <class DT> __device__ inline u32x2 pack_acc(f32x4 a, float f) {
 // g the neighbour's half of the odd tile.  Half as many stores, and one instruction writes whole 64-byte pieces of
 // a row instead of 32-byte halves that the other instruction completes later.
 template <int C, int AUX>
-__device__ inline void store_tile(Rsrc dst, int row_byte, const u32x2 (&w)[C / 16], int g) {
+__device__ inline void store_tile(Rsrc dst, int row_byte, const u32x2 (&w)[C / 16], int g, int width) {
     constexpr int CT = C / 16;
     if constexpr (CT == 1) {
-        __builtin_amdgcn_raw_buffer_store_b64(w[0], dst, row_byte + g * 8, 0, AUX);
+        __builtin_amdgcn_raw_buffer_store_b64(w[0], dst, g * 8 < width ? row_byte + g * 8 : kNowhere, 0, AUX);
     } else {
 #pragma unroll
         for (int p = 0; p < CT / 2; ++p) {
             const u32x2 lo = __builtin_amdgcn_permlane16_swap(w[2 * p].x, w[2 * p + 1].x, false, false);
             const u32x2 hi = __builtin_amdgcn_permlane16_swap(w[2 * p].y, w[2 * p + 1].y, false, false);
             const u32x4 v = {lo.x, hi.x, lo.y, hi.y};
-            __builtin_amdgcn_raw_buffer_store_b128(v, dst, row_byte + (2 * p + (g & 1)) * 32 + (g >> 1) * 16, 0, AUX);
+            const int at = (2 * p + (g & 1)) * 32 + (g >> 1) * 16;      // channels past head_dim are not stored
+            __builtin_amdgcn_raw_buffer_store_b128(v, dst, at < width ? row_byte + at : kNowhere, 0, AUX);
         }
     }
 }
 template <int C>
-__device__ inline void store_tile(Rsrc dst, int row_byte, const u32x2 (&w)[C / 16], int g, bool stream) {
+__device__ inline void store_tile(Rsrc dst, int row_byte, const u32x2 (&w)[C / 16], int g, bool stream, int width) {
     if (stream)
-        store_tile<C, kStoreAux>(dst, row_byte, w, g);
+        store_tile<C, kStoreAux>(dst, row_byte, w, g, width);
     else
-        store_tile<C, 0>(dst, row_byte, w, g);
+        store_tile<C, 0>(dst, row_byte, w, g, width);
 }
 
 // ---- window slots of a lane ------------------------------------------------------
@@ -374,8 +379,11 @@ inline Split make_split(int64_t B, int64_t T, int max_tiles) {
 struct Strides {
     int64_t sample, head;   // from one sample / head to the next
     int pitch;              // from one row to the next
+    int width;              // bytes of a row that exist: 2 * head_dim
 };
-inline Strides byte_strides(const Layout &l) { return Strides{2 * l.sample, 2 * l.head, (int)(2 * l.row)}; }
+inline Strides byte_strides(const Layout &l, const Geom &g) {
+    return Strides{2 * l.sample, 2 * l.head, (int)(2 * l.row), 2 * g.C};
+}
 // Offsets inside one sequence are 32-bit: the rows of a sequence, plus the halo rows the copies ask for
 // beyond its end, must span less than 2^30 bytes.
 inline bool strides_ok(const Layout &l, const Geom &g) { return l.row >= g.C && g.T + 96 <= (1 << 29) / l.row; }
@@ -433,7 +441,7 @@ inline bool allow_lds(K kern, size_t bytes) {
 // Number of virtual key blocks the kernels need, 0 if the shape is not covered.
 inline int window_blocks(const Geom &g) {
     const int R = g.W - 1 - g.L;
-    if (g.C != 16 && g.C != 32 && g.C != 64 && g.C != 128) return 0;
+    if (g.C > 128) return 0;               // head_dim is run at the next of 16, 32, 64, 128, zero-padded
     if (g.T > (1 << 29) / g.C) return 0;   // per-sequence byte offsets stay in 31 bits
     if (15 + g.W <= 32) return 2;
     if (g.L <= 16 && R <= 16 && g.W <= 32) return 3;
@@ -450,17 +458,20 @@ inline int window_shift(const Geom &g) {
     return s <= 16 - R ? s : g.L;
 }
 
+// The kernels' C for a head_dim: the next of 16, 32, 64, 128 (0 above).
+inline int padded_width(int head_dim) { return head_dim <= 16 ? 16 : head_dim <= 32 ? 32 : head_dim <= 64 ? 64 : head_dim <= 128 ? 128 : 0; }
+
 #define NA1D_MFMA_DISPATCH(FN, ...)                                            \
     do {                                                                       \
         if (dtype == NA1D_BF16) {                                              \
-            switch (g.C) {                                                     \
+            switch (padded_width(g.C)) {                                                     \
                 case 16: return FN<BF16, 16>(__VA_ARGS__);                     \
                 case 32: return FN<BF16, 32>(__VA_ARGS__);                     \
                 case 64: return FN<BF16, 64>(__VA_ARGS__);                     \
                 case 128: return FN<BF16, 128>(__VA_ARGS__);                   \
             }                                                                  \
         } else {                                                               \
-            switch (g.C) {                                                     \
+            switch (padded_width(g.C)) {                                                     \
                 case 16: return FN<FP16, 16>(__VA_ARGS__);                     \
                 case 32: return FN<FP16, 32>(__VA_ARGS__);                     \
                 case 64: return FN<FP16, 64>(__VA_ARGS__);                     \

@@ -20,7 +20,7 @@ struct BandCover {
 };
 inline BandCover band_cover(const Geom &g) {
     BandCover c{0, 0, 0};
-    if (g.C != 16 && g.C != 32 && g.C != 64 && g.C != 128) return c;
+    if (g.C > 128) return c;             // head_dim is run at the next of 16, 32, 64, 128, zero-padded
     if (g.T > (1 << 29) / g.C || g.T > (1 << 29) / (4 * g.W) || g.W > NA1D_MAX_WINDOW) return c;
     c.nbv = std::max(2, (15 + g.W + 15) / 16);
     const int R = g.W - 1 - g.L, rows = std::max(1, 128 / (2 * g.C));
@@ -61,10 +61,10 @@ __device__ inline float score_at(LDS_PTR(float) rows, int row, int j, int W) {  
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__restrict__ kb, uint32_t items, int T,
-          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift) {
+          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift, int pitch) {
     using LL = Lds<C>;
     constexpr int MT = kBandMaxTiles;
-    fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic, shift);
+    fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
     // dynamic LDS: K region of kt tiles starting sb tiles before the strip, Q region of nt tiles, one 16 x W fp32
     // tile per wave
     const int sb = (shift + 15) >> 4, kt = nt - 1 + NBV + ((shift & 15) ? 1 : 0);
@@ -81,12 +81,12 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
 
-    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    const int64_t seq_off = (int64_t)b * T * pitch;      // packed rows of head_dim = pitch / 2 channels
     {
-        const int key_bytes = min(T, 16 * (i0 - sb + kt)) * 2 * C, qry_bytes = min(T, 16 * i1) * 2 * C;
-        const int lane_off = direct_lane_offset<C>(wave, lane);
-        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off);
-        stage_direct<C, MT, kReadShared>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off);
+        const int key_bytes = min(T, 16 * (i0 - sb + kt)) * pitch, qry_bytes = min(T, 16 * i1) * pitch;
+        const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
+        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off, pitch);
+        stage_direct<C, MT, kReadShared>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off, pitch);
     }
     const Rsrc as = make_rsrc(attn + (int64_t)b * T * W, T * W * 4);
     RowLane<C> k_lane, q_lane;
@@ -134,11 +134,11 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ v, uint32_t items, int T,
-          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift) {
+          int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift, int pitch) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = kBandMaxTiles;
-    fetch_args_now(out, attn, v, items, T, W, L, tiles, nt, strips, strips_magic, shift);
+    fetch_args_now(out, attn, v, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
     // dynamic LDS: V region of kt tiles starting sb tiles before the strip, score rows of the strip (nt*16 x W fp32)
     const int sb = (shift + 15) >> 4, kt = nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -153,14 +153,14 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
     const int i0 = strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
 
-    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    const int64_t seq_off = (int64_t)b * T * pitch;      // packed rows of head_dim = pitch / 2 channels
     {
-        const int key_bytes = min(T, 16 * (i0 - sb + kt)) * 2 * C;
+        const int key_bytes = min(T, 16 * (i0 - sb + kt)) * pitch;
         stage_direct<C, MT + NBV, kReadShared>(make_rsrc(v + seq_off, key_bytes), 16 * (i0 - sb), v_lds, kt, wave,
-                                               direct_lane_offset<C>(wave, lane));
+                                               direct_lane_offset<C>(wave, lane, pitch, pitch), pitch);
         stage_scores<NBV>(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, s_lds, nt, W, wave, lane);
     }
-    const Rsrc os = make_rsrc(out + seq_off, T * 2 * C);
+    const Rsrc os = make_rsrc(out + seq_off, T * pitch);
     TrLane<C> v_lane;
     v_lane.init(16 * sb - shift, lane);
     wait_direct();
@@ -186,7 +186,7 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], 1.f);
-        store_tile<C, kStoreAux>(os, qrow * (2 * C), ow, g);
+        store_tile<C>(os, qrow * pitch, ow, g, stores_whole_lines(pitch, C, 0), pitch);
     }
 }
 
@@ -196,11 +196,11 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
 template <class DT, int C, int NBV>
 __global__ void __launch_bounds__(kThreads)
 gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__restrict__ x, uint32_t items,
-              int T, int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift) {
+              int T, int W, int L, int tiles, int nt, int strips, uint32_t strips_magic, int shift, int pitch) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = kBandMaxTiles;
-    fetch_args_now(out, attn, x, items, T, W, L, tiles, nt, strips, strips_magic, shift);
+    fetch_args_now(out, attn, x, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
     // Key block kp (rows 16*kp - shift ...) is virtual block vb of query tile kp - vb, so the blocks that touch the
     // strip's rows need the query tiles i0 - hb .. i1 - 1 + ha.  Dynamic LDS: their x rows (qtiles tiles) and their
     // score rows (qtiles*16 x W fp32)
@@ -218,17 +218,17 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     const int g = lane >> 4, n = lane & 15;
     const int q0 = i0 - hb;                                            // first query tile needed
 
-    const int64_t seq_off = (int64_t)b * T * (2 * C);
+    const int64_t seq_off = (int64_t)b * T * pitch;      // packed rows of head_dim = pitch / 2 channels
     {
         const int rows_hi = min(T, 16 * (q0 + qtiles));
-        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(x + seq_off, rows_hi * 2 * C), 16 * q0, x_lds, qtiles, wave,
-                                               direct_lane_offset<C>(wave, lane));
+        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(x + seq_off, rows_hi * pitch), 16 * q0, x_lds, qtiles, wave,
+                                               direct_lane_offset<C>(wave, lane, pitch, pitch), pitch);
         stage_scores<NBV>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), 16 * q0 * W, s_lds, qtiles, W, wave, lane);
     }
     TrLane<C> x_tr;
     x_tr.init(0, lane);
     const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
-    const Rsrc os = make_rsrc(out + seq_off + (int64_t)row_lo * (2 * C), (row_hi - row_lo) * 2 * C);
+    const Rsrc os = make_rsrc(out + seq_off + (int64_t)row_lo * pitch, (row_hi - row_lo) * pitch);
     wait_direct();
     __syncthreads();
 
@@ -251,11 +251,11 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(xt + x_tr.off[ct]), pb, acc[ct]);
         }
-        const int row_off = (16 * (kp - i0) - shift + n) * (2 * C);     // outside the strip -> dropped
+        const int row_off = (16 * (kp - i0) - shift + n) * pitch;       // outside the strip -> dropped
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(acc[ct], 1.f);
-        store_tile<C>(os, row_off, ow, g, stores_whole_lines(2 * C, C, shift));
+        store_tile<C>(os, row_off, ow, g, stores_whole_lines(pitch, C, shift), pitch);
     }
 }
 
@@ -284,7 +284,7 @@ int launch_qk_n(float *attn, const void *a, const void *b, const Geom &g, const 
     const size_t lds = lds_of(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>(attn, (const char *)a, (const char *)b, (uint32_t)sp.items, (int)g.T,
-                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift);
+                                                   g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift, 2 * g.C);
     return launch_status();
 }
 
@@ -301,7 +301,7 @@ int launch_av_n(void *out, const float *attn, const void *v, const Geom &g, cons
     const size_t lds = lds_of(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)v, (uint32_t)sp.items, (int)g.T, g.W,
-                                                   g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift);
+                                                   g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift, 2 * g.C);
     return launch_status();
 }
 
@@ -317,7 +317,7 @@ int launch_gather_n(void *out, const float *attn, const void *x, const Geom &g, 
     const size_t lds = lds_of(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)x, (uint32_t)sp.items, (int)g.T, g.W,
-                                                   g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift);
+                                                   g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift, 2 * g.C);
     return launch_status();
 }
 

@@ -17,7 +17,7 @@ struct WideCover {
 };
 inline WideCover wide_cover(const Geom &g) {
     WideCover c{0, 0};
-    if (g.C != 16 && g.C != 32 && g.C != 64 && g.C != 128) return c;
+    if (g.C > 128) return c;             // head_dim is run at the next of 16, 32, 64, 128, zero-padded
     if (g.T > (1 << 29) / g.C || g.W > NA1D_MAX_WINDOW) return c;
     c.nbv = (15 + g.W + 15) / 16;
     if (c.nbv < 3) c.nbv = 3;
@@ -51,7 +51,7 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
     constexpr int CT = C / 16;
     constexpr int MT = Strip<C>::kMaxTiles;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
-                   in.sample, in.head, in.pitch, outl.sample, outl.head, outl.pitch, shift);
+                   in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift);
     // dynamic LDS (launch_wide_fwd): K and V regions of kt tiles starting sb tiles before the strip, Q region of nt
     // tiles, kBiasSlots bias floats
     const int sb = (shift + 15) >> 4;                        // whole tiles in front of the strip
@@ -77,7 +77,7 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
     const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
     const bool out_whole_lines = stores_whole_lines(outl.pitch, C, 0);
     {
-        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch);
+        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
         stage_direct<C, MT + NBV, kReadShared>(ks, 16 * (i0 - sb), k_lds, kt, wave, lane_off, in.pitch);
         stage_direct<C, MT, kReadShared>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
         stage_direct<C, MT + NBV, kReadShared>(vs, 16 * (i0 - sb), v_lds, kt, wave, lane_off, in.pitch);
@@ -158,7 +158,7 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
-        store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines);   // rows past T are dropped by the store
+        store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines, outl.width);   // rows past T are dropped by the store
         if (g == 0)
             __builtin_amdgcn_raw_buffer_store_b32(
                 __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2), ls, qrow * 4, 0, 0);
@@ -177,7 +177,7 @@ int launch_wide_fwd_n(void *out, float *lse, const void *q, const void *k, const
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
-                  div_magic(sp.strips), div_magic(g.H), byte_strides(in), byte_strides(outl), shift);
+                  div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), shift);
     return launch_status();
 }
 
@@ -238,8 +238,8 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
     constexpr int CT = C / 16;
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
-                   kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, outl.sample, outl.head,
-                   outl.pitch, shift);
+                   kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width, outl.sample,
+                   outl.head, outl.pitch, outl.width, shift);
     const int hb = NBV - 1 - (shift >> 4), ha = (shift + 15) >> 4;
     const int qtiles = nt + hb + ha;                        // query-side tiles, <= kWideQueryTiles
     const int ktiles = qtiles + NBV - 1;                    // key-side tiles: whole virtual blocks
@@ -272,8 +272,8 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
         const Rsrc ks = make_rsrc(k + in_off, key_rows * in.pitch), vs = make_rsrc(v + in_off, key_rows * in.pitch);
         const Rsrc qs = make_rsrc(q + in_off, qry_rows * in.pitch), gs = make_rsrc(dout + out_off, qry_rows * outl.pitch);
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
-        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch);
-        const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch);
+        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
+        const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch, outl.width);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * q0 + tid) * 4, 0, 0, 0);
         constexpr int KT = kWideQueryTiles + NBV - 1;
         stage_direct<C, KT, kReadShared>(ks, 16 * q0 - shift, k_lds, ktiles, wave, lane_off, in.pitch);
@@ -371,7 +371,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
         u32x2 qw[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[ct], scale);
-        store_tile<C>(dqs, qrow * in.pitch, qw, g, dq_whole_lines);
+        store_tile<C>(dqs, qrow * in.pitch, qw, g, dq_whole_lines, in.width);
     }
 
     // d rpb.  Register (vb, r) of lane (n, g) holds key a = 4g + r of block vb against query n: slot
@@ -447,8 +447,8 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
             kw[ct] = pack_acc<DT>(acck[ct], scale);
             vw[ct] = pack_acc<DT>(accv[ct], 1.f);
         }
-        store_tile<C>(dks, row_off, kw, g, whole_lines);
-        store_tile<C>(dvs, row_off, vw, g, whole_lines);
+        store_tile<C>(dks, row_off, kw, g, whole_lines, in.width);
+        store_tile<C>(dvs, row_off, vw, g, whole_lines, in.width);
     }
 
     if (drpb && tid < W) {              // rsum was complete at the barriers before pass 2
@@ -484,7 +484,7 @@ int launch_wide_bwd_n(void *dq, void *dk, void *dv, float *drpb, const void *q, 
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, kv_bytes, div_magic(sp.strips), div_magic(g.H),
-                  byte_strides(in), byte_strides(outl), c.shift);
+                  byte_strides(in, g), byte_strides(outl, g), c.shift);
     return launch_status();
 }
 

@@ -82,7 +82,7 @@ def test_fused_entry_points_validate():
     w = lib.na1d_fused_backward_workspace_bytes
     assert w(4096, 16, 100, 16, 27, 13, 0) == 4096 * 32 * 4      # one 32-float row per work item
     assert w(1024, 8, 300, 32, 15, 7, 1) > 0
-    assert w(4, 2, 8, 24, 5, 2, 0) == 0                          # generic kernel: no workspace
+    assert w(4, 2, 8, 136, 5, 2, 0) == 0                         # generic kernel: no workspace
     assert w(4, 3, 8, 16, 5, 2, 0) == -5 and w(4, 2, 8, 16, 99, 2, 0) == -4
 
 
@@ -100,7 +100,7 @@ def test_strided_entry_points_validate():
     assert f(*args(os=S(-256, 16, 32))) == -5
     assert f(*args(C=20)) == -3 and f(*args(W=99)) == -4 and f(*args(N=-1)) == -5
     assert f(*args(N=0)) == 0                        # nothing to do
-    assert f(*args(C=24, qs=S(8 * 3 * 2 * 24, 24, 3 * 2 * 24), os=S(8 * 2 * 24, 24, 48))) == -8   # no strided kernel for C=24
+    assert f(*args(C=136, qs=S(8 * 3 * 2 * 136, 136, 3 * 2 * 136), os=S(8 * 2 * 136, 136, 272))) == -8   # no strided kernel above 128
     b = lib.na1d_fused_backward_strided
     bargs = lambda **kw: [ok, ok, ok, None, ok, ok, ok, kw.get("g", ok), kw.get("lse", ok), None, None, 2, 2, 8, 16, 5, 2,
                           1.0, 0, kw.get("qs", qkv), out, kw.get("ws", None), 64, None]

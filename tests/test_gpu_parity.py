@@ -23,6 +23,7 @@ SHAPES = [
     (2, 5, 8, 5, 4), (1, 1, 8, 3, 1), (2, 40, 24, 11, 5), (2, 33, 40, 8, 3), (1, 100, 16, 27, 13),
     (2, 100, 128, 80, 39), (2, 17, 16, 80, 0), (2, 130, 64, 7, 3), (4, 300, 32, 15, 7), (3, 65, 16, 27, 26),
     (2, 47, 48, 33, 16), (2, 64, 16, 27, 13), (1, 16, 32, 15, 7), (2, 15, 64, 7, 3), (2, 250, 16, 9, 8),
+    (2, 70, 56, 27, 13), (1, 90, 72, 15, 7), (2, 50, 96, 40, 20), (1, 33, 120, 7, 3), (2, 40, 136, 9, 4),
 ]
 
 
@@ -135,7 +136,8 @@ FUSED_GEOMS = [  # (N, H, T, C, W, left)
     (2, 4, 60, 16, 27, 13), (3, 2, 33, 32, 15, 7), (2, 2, 9, 64, 7, 3), (2, 3, 21, 24, 8, 3), (1, 1, 1, 8, 3, 1),
     (2, 2, 5, 16, 27, 13), (1, 2, 100, 16, 27, 0), (1, 2, 100, 16, 27, 26), (2, 1, 70, 40, 80, 40), (2, 16, 100, 16, 27, 13),
     (3, 4, 150, 16, 27, 13), (2, 8, 300, 32, 15, 7), (4, 4, 200, 64, 7, 3), (1, 2, 129, 128, 5, 2), (2, 2, 48, 16, 1, 0),
-    (1, 4, 257, 32, 40, 7), (1, 2, 31, 64, 33, 20),
+    (1, 4, 257, 32, 40, 7), (1, 2, 31, 64, 33, 20), (2, 2, 90, 56, 27, 13), (1, 2, 75, 72, 15, 7), (2, 1, 60, 96, 50, 25),
+    (1, 2, 40, 120, 7, 3), (2, 2, 100, 8, 27, 13), (1, 2, 50, 136, 9, 4),
 ]
 
 
