@@ -165,6 +165,26 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb,
                                 void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * Dense ("global") attention over whole sequences, forward and backward: replaces the body of the reference's
+ * GlobalAttention.forward between the head split and the head merge (models/PCF_NATransformer.py:199-221),
+ *     attn = softmax((q * scale) @ k^T + mask);  out = attn @ v
+ * with the mask of get_attn_mask_global (models/PCF_NATransformer.py:406-414) built on the fly from t_valid:
+ * -100 is added where the query row or the key column is >= t_valid[sample] (NULL: nothing is padded).
+ * q, k, v, out and the gradients are packed [B, T, C] with B = samples * H, head fastest inside a sample;
+ * lse [B, T] fp32 (natural log; may be NULL in the forward when no backward follows).  The probabilities are never
+ * written to memory.  The backward needs a workspace of na1d_global_backward_workspace_bytes() bytes (one fp32 per
+ * row: rowsum(dout * out)) and writes every gradient exactly once, so it is deterministic.
+ * C % 8 == 0; C > 128 returns NA1D_ERR_UNSUPPORTED.  Attention dropout (the reference's attn_drop) is not applied:
+ * the reference's configurations set it to 0.
+ */
+int na1d_global_forward(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
+                        int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, void *stream);
+int na1d_global_backward(void *dq, void *dk, void *dv, const void *q, const void *k, const void *v, const void *out,
+                         const void *dout, const float *lse, const int32_t *t_valid, int64_t B, int64_t H, int64_t T,
+                         int64_t C, float scale, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int dtype);
+
+/*
  * Profiling hook; no counterpart in the reference.  From this call on, the matrix-core fused kernels that the
  * CALLING THREAD launches record `start` just before and `stop` just after the kernel itself (hipEvent_t handles,
  * recorded by hipExtLaunchKernel: the dispatch's own begin and end, i.e. what a profiler's kernel trace reports,

@@ -17,13 +17,16 @@ the autograd wiring around its kernels:
 * inverse-neighbourhood gather (P3)            na1d_tensorcore/bf16_ana1d_kernel.cu:457-459,
                                                na1d_tensorcore/nattn.py:46-54,69-78
 * dilation > 1 (CPU only in the reference)     models/PCF_NATransformer.py:101-116,158-159,169-170
+* dense attention of the global layers         models/PCF_NATransformer.py:215-221, mask :406-414
 
 What pins each function (see tests/test_oracle_pins.py): brute-force index
 loops on tiny shapes, W=1 row dots, the dense ``q @ k^T`` embedding for
 ``L=T-1, W=2T-1``, ``k=1`` zero-fill, one-hot / uniform probabilities for P2,
 the exact adjoint identities between P1/P2/P3, closed-form masks, library
-softmax on the valid slots, and ``torch.autograd.gradcheck`` in fp64.  No
-function here is "parity unpinned".
+softmax on the valid slots, and ``torch.autograd.gradcheck`` in fp64; the dense
+attention by index loops, ``F.scaled_dot_product_attention`` with the same mask,
+the closed-form mask, the full-window NA1D it must agree with, and gradcheck.
+No function here is "parity unpinned".
 
 Layout everywhere: ``q, k, v : [B, T, C]`` with ``B = N * H`` (batch major,
 head minor), scores / probabilities ``[B, T, W]``; slot ``j`` of query ``t``
@@ -173,6 +176,41 @@ def na1d_backward_formulas(q, k, v, do, W, left, rpb=None, padding=None, num_hea
     dk = inverse_gather(ds, q, W, left)
     drpb = ds.view(B // num_heads, num_heads, T, W).sum(dim=(0, 2))
     return dq, dk, dv, drpb
+
+
+# --------------------------------------------------------------------------
+# dense attention of the global layers
+# --------------------------------------------------------------------------
+def global_mask(T, padding=None, dtype=torch.float32):
+    """[N,T,T] additive mask: -100 where the query row or the key column is padded, one fill (never -200).
+    models/PCF_NATransformer.py:406-414.
+    """
+    if padding is None:
+        padding = torch.zeros(1, dtype=torch.int64)
+    padding = torch.as_tensor(padding, dtype=torch.int64).reshape(-1)
+    t_valid = (T - padding).view(-1, 1, 1)
+    t = torch.arange(T)
+    bad = (t.view(1, T, 1) >= t_valid) | (t.view(1, 1, T) >= t_valid)
+    return torch.zeros(bad.shape, dtype=dtype).masked_fill(bad, MASK_VALUE)
+
+
+def global_forward(q, k, v, scale, padding=None, num_heads=1):
+    """``softmax(q k^T * scale + mask) v`` per head: returns ``(O, P, LSE)``.
+    models/PCF_NATransformer.py:215-221 (``q * scale`` is applied here to the product instead).
+    """
+    B, T, _ = q.shape
+    z = torch.einsum("btc,buc->btu", q, k) * scale
+    m = global_mask(T, padding, dtype=z.dtype)                    # [N or 1, T, T]
+    z = (z.view(B // num_heads, num_heads, T, T) + m.unsqueeze(1)).view(B, T, T)
+    p = torch.softmax(z, dim=-1)
+    return torch.einsum("btu,buc->btc", p, v), p, torch.logsumexp(z, dim=-1)
+
+
+def global_backward(q, k, v, do, scale, padding=None, num_heads=1):
+    """``(dq, dk, dv)`` by ``torch.autograd`` through :func:`global_forward`."""
+    leaves = [x.detach().clone().requires_grad_(True) for x in (q, k, v)]
+    o, _, _ = global_forward(*leaves, scale, padding, num_heads)
+    return torch.autograd.grad(o, leaves, do)
 
 
 # --------------------------------------------------------------------------

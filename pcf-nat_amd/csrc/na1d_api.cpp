@@ -229,6 +229,33 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb, const
                           (float *)workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
 }
 
+int na1d_global_forward(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
+                        int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, void *stream) {
+    NA1D_CHECK(out, q, k, B, T, C, 1, 0, H, dtype, g);
+    if (!v) return NA1D_ERR_NULL;
+    if (misaligned(v)) return NA1D_ERR_ALIGN;
+    return na1d::mfma::global_fwd(out, lse, q, k, v, t_valid, g, scale, dtype, (hipStream_t)stream);
+}
+
+int na1d_global_backward(void *dq, void *dk, void *dv, const void *q, const void *k, const void *v, const void *out,
+                         const void *dout, const float *lse, const int32_t *t_valid, int64_t B, int64_t H, int64_t T,
+                         int64_t C, float scale, int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+    NA1D_CHECK(dq, q, k, B, T, C, 1, 0, H, dtype, g);
+    if (!dk || !dv || !v || !out || !dout || !lse || !workspace) return NA1D_ERR_NULL;
+    if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout) || misaligned(workspace))
+        return NA1D_ERR_ALIGN;
+    if (workspace_bytes < g.B * g.T * (int64_t)sizeof(float)) return NA1D_ERR_SHAPE;
+    return na1d::mfma::global_bwd(dq, dk, dv, (float *)workspace, q, k, v, out, dout, lse, t_valid, g, scale, dtype,
+                                  (hipStream_t)stream);
+}
+
+int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int dtype) {
+    Geom g;
+    const int st = check_shape(B, T, C, 1, 0, H, dtype, g);
+    if (st < 0) return st;
+    return st > 0 ? 0 : g.B * g.T * (int64_t)sizeof(float);
+}
+
 int na1d_profile_events(void *start, void *stop) {
     na1d::LaunchEvents &ev = na1d::launch_events();
     ev.start = (hipEvent_t)start;

@@ -126,6 +126,12 @@ int wide_fwd(void *out, float *lse, const void *q, const void *k, const void *v,
 int wide_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v, const void *dout,
              const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g, const Layout &in,
              const Layout &out_layout, float scale, int dtype, hipStream_t s);
+// Dense attention over whole sequences (the models' global layers); g.W and g.L are not used.
+int global_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
+               const Geom &g, float scale, int dtype, hipStream_t s);
+int global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q, const void *k, const void *v, const void *out,
+               const void *dout, const float *lse, const int32_t *t_valid, const Geom &g, float scale, int dtype,
+               hipStream_t s);
 }  // namespace mfma
 
 }  // namespace na1d

@@ -1,0 +1,444 @@
+// Dense ("global") attention of the models' two global layers on the matrix cores (gfx950):
+//   P = softmax(q k^T * scale + M),  O = P v,   M[t, u] = -100 where row t or column u is padded
+// (models/PCF_NATransformer.py:199-221 with the mask of :406-414).  Flash-attention style, built
+// from the tile machinery of na1d_mfma_core.h: S^T tiles of 16 keys x 16 queries, an online
+// softmax whose row statistics are lane-local up to a reduction over the four lane groups, and
+// the rounded probabilities fed straight back as the B operand of O^T += V^T P^T.
+//
+// Forward: a workgroup owns 4 query tiles (one per wave) and walks the keys in chunks of 4 tiles
+// that all four waves share through LDS.
+// Backward: one kernel per query strip computes delta = rowsum(dO * O) and dQ, walking the keys;
+// a second per key strip computes dK and dV, walking the queries with Q and K swapped in the
+// score product so that the probabilities come out as "lane = key, registers = queries", which
+// is the B operand of dV^T += dO^T P and dK^T += Q^T dS.  No atomics, every output written once.
+#include "na1d_mfma_core.h"
+
+namespace na1d {
+namespace mfma {
+
+constexpr int kStripTiles = 4;      // tiles per strip (one per wave) and per chunk
+static_assert(kStripTiles == kWaves, "one tile of the strip per wave");
+
+// Two 16-bit values of a register as floats.
+template <class DT> __device__ inline f32x2 unpack2(uint32_t w);
+template <> __device__ inline f32x2 unpack2<BF16>(uint32_t w) {
+    return f32x2{__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u)};
+}
+template <> __device__ inline f32x2 unpack2<FP16>(uint32_t w) {
+    return __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2);
+}
+// sum over this lane's channels of a[c] * b[c] for two row operands
+template <class DT, int C>
+__device__ inline float dot_lane(const RowOperand<C> &a, const RowOperand<C> &b) {
+    float acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < RowOperand<C>::k32; ++s)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const f32x2 x = unpack2<DT>(a.w32[s][i]), y = unpack2<DT>(b.w32[s][i]);
+            acc = __builtin_fmaf(x.x, y.x, __builtin_fmaf(x.y, y.y, acc));
+        }
+    if (RowOperand<C>::k16)
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const f32x2 x = unpack2<DT>(a.w16[0][i]), y = unpack2<DT>(b.w16[0][i]);
+            acc = __builtin_fmaf(x.x, y.x, __builtin_fmaf(x.y, y.y, acc));
+        }
+    return acc;
+}
+
+struct GlobalArgs {
+    int T, H, strips;            // strips of kStripTiles tiles per sequence
+    uint32_t strips_magic, heads_magic;
+    int pitch;                   // bytes per row = 2 * head_dim (packed rows)
+    float scale;
+};
+
+// =============================================================================
+// Forward
+// =============================================================================
+template <class DT, int C>
+__global__ void __launch_bounds__(kThreads)
+global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
+                  const char *__restrict__ k, const char *__restrict__ v, const int32_t *__restrict__ t_valid,
+                  uint32_t items, GlobalArgs a) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16;
+    fetch_args_now(out, lse, q, k, v, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic, a.pitch, a.scale);
+    constexpr int kStep = region_bytes<C>(kStripTiles);
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 3 * kStep bytes
+    LDS_PTR(char) q_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) k_lds = q_lds + kStep;
+    LDS_PTR(char) v_lds = k_lds + kStep;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, n = lane & 15;
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = div_by(item, a.strips, a.strips_magic);
+    const int strip = (int)(item - b * a.strips);
+    const uint32_t sample = div_by(b, a.H, a.heads_magic);
+    const int T = a.T, tiles = (T + 15) >> 4;
+    const int qt = kStripTiles * strip + wave;              // this wave's query tile
+    const int qrow = 16 * qt + n;
+
+    const int64_t seq_off = (int64_t)b * T * a.pitch;
+    const Rsrc qs = make_rsrc(q + seq_off, T * a.pitch), ks = make_rsrc(k + seq_off, T * a.pitch);
+    const Rsrc vs = make_rsrc(v + seq_off, T * a.pitch), os = make_rsrc(out + seq_off, T * a.pitch);
+    const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
+    const int lane_off = direct_lane_offset<C>(wave, lane, a.pitch, a.pitch);
+    int tv = T;
+    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
+    const bool row_masked = qrow >= tv;
+
+    RowLane<C> row_lane;
+    TrLane<C> tr_lane;
+    row_lane.init(0, lane);
+    tr_lane.init(0, lane);
+
+    stage_direct<C, kStripTiles, kReadShared>(qs, 16 * kStripTiles * strip, q_lds, kStripTiles, wave, lane_off, a.pitch);
+    float m = kNegInf, l = 0.f;
+    f32x4 o[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    RowOperand<C> qop;
+
+    for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
+        if (c0) __syncthreads();                            // every wave is done with the previous chunk
+        stage_direct<C, kStripTiles, kReadShared>(ks, 16 * c0, k_lds, kStripTiles, wave, lane_off, a.pitch);
+        stage_direct<C, kStripTiles, kReadShared>(vs, 16 * c0, v_lds, kStripTiles, wave, lane_off, a.pitch);
+        wait_direct();
+        __syncthreads();
+        if (c0 == 0) read_rows<C>(qop, q_lds + wave * LL::kTileBytes, row_lane);
+        const int nk = min(kStripTiles, tiles - c0);        // key tiles in this chunk
+        float z[kStripTiles][4];
+        float mc = kNegInf;
+#pragma unroll
+        for (int kt = 0; kt < kStripTiles; ++kt) {
+            if (kt < nk) {
+                RowOperand<C> kop;
+                read_rows<C>(kop, k_lds + kt * LL::kTileBytes, row_lane);
+                const f32x4 s = dot_rows_mma<DT, C>(kop, qop);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = 16 * (c0 + kt) + 4 * g + r;
+                    float zz = s[r] * scale2 + ((key >= tv || row_masked) ? mask2 : 0.f);
+                    z[kt][r] = key < T ? zz : kNegInf;      // rows past the sequence do not exist
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) z[kt][r] = kNegInf;
+            }
+            mc = max3(mc, max2(z[kt][0], z[kt][1]), max2(z[kt][2], z[kt][3]));
+        }
+        const float m_new = max2(m, xor_max(mc));           // finite: key 16*c0 exists
+        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+        float part = 0.f;
+        u32x2 pb[kStripTiles];
+#pragma unroll
+        for (int kt = 0; kt < kStripTiles; ++kt) {
+            float p[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                p[r] = __builtin_amdgcn_exp2f(z[kt][r] - m_new);
+                part += p[r];
+            }
+            pb[kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+        }
+        l = l * alpha + xor_sum(part);
+        m = m_new;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[ct] = o[ct] * alpha;
+#pragma unroll
+        for (int kt = 0; kt < kStripTiles; ++kt) {
+            if (kt >= nk) continue;
+            LDS_PTR(char) blk = v_lds + kt * LL::kTileBytes;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr(blk + tr_lane.off[ct]), pb[kt], o[ct]);
+        }
+    }
+    if (qt >= tiles) return;                                // after the last barrier
+    const float inv = __builtin_amdgcn_rcpf(l);
+    u32x2 ow[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
+    store_tile<C>(os, qrow * a.pitch, ow, g, stores_whole_lines(a.pitch, C, 0), a.pitch);   // rows past T are dropped
+    if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint((m + __builtin_amdgcn_logf(l)) * kLn2), ls, qrow * 4, 0, 0);
+}
+
+// =============================================================================
+// Backward, query side: delta = rowsum(dO * O) (written to `delta`) and dQ
+// =============================================================================
+template <class DT, int C>
+__global__ void __launch_bounds__(kThreads)
+global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *__restrict__ q,
+                 const char *__restrict__ k, const char *__restrict__ v, const char *__restrict__ out,
+                 const char *__restrict__ dout, const float *__restrict__ lse, const int32_t *__restrict__ t_valid,
+                 uint32_t items, GlobalArgs a) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16;
+    constexpr int kStep = region_bytes<C>(kStripTiles);
+    fetch_args_now(dq, delta, q, k, v, out, dout, lse, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic,
+                   a.pitch, a.scale);
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 5 * kStep bytes
+    LDS_PTR(char) q_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) g_lds = q_lds + kStep;                    // dO
+    LDS_PTR(char) o_lds = g_lds + kStep;
+    LDS_PTR(char) k_lds = o_lds + kStep;
+    LDS_PTR(char) v_lds = k_lds + kStep;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, n = lane & 15;
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = div_by(item, a.strips, a.strips_magic);
+    const int strip = (int)(item - b * a.strips);
+    const uint32_t sample = div_by(b, a.H, a.heads_magic);
+    const int T = a.T, tiles = (T + 15) >> 4;
+    const int qt = kStripTiles * strip + wave;
+    const int qrow = 16 * qt + n;
+
+    const int64_t seq_off = (int64_t)b * T * a.pitch;
+    const Rsrc qs = make_rsrc(q + seq_off, T * a.pitch), ks = make_rsrc(k + seq_off, T * a.pitch);
+    const Rsrc vs = make_rsrc(v + seq_off, T * a.pitch), os = make_rsrc(out + seq_off, T * a.pitch);
+    const Rsrc gs = make_rsrc(dout + seq_off, T * a.pitch), dqs = make_rsrc(dq + seq_off, T * a.pitch);
+    const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4), ds = make_rsrc(delta + (int64_t)b * T, T * 4);
+    const int lane_off = direct_lane_offset<C>(wave, lane, a.pitch, a.pitch);
+    int tv = T;
+    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
+    const bool row_masked = qrow >= tv;
+    const float lse2 = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ls, qrow * 4, 0, 0)) * kLog2e;
+
+    RowLane<C> row_lane;
+    TrLane<C> tr_lane;
+    row_lane.init(0, lane);
+    tr_lane.init(0, lane);
+
+    const int row0 = 16 * kStripTiles * strip;
+    stage_direct<C, kStripTiles, kReadShared>(qs, row0, q_lds, kStripTiles, wave, lane_off, a.pitch);
+    stage_direct<C, kStripTiles, kReadShared>(gs, row0, g_lds, kStripTiles, wave, lane_off, a.pitch);
+    stage_direct<C, kStripTiles, kReadShared>(os, row0, o_lds, kStripTiles, wave, lane_off, a.pitch);
+    f32x4 acc[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    RowOperand<C> qop, gop;
+    float dl = 0.f;
+
+    for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
+        if (c0) __syncthreads();
+        stage_direct<C, kStripTiles, kReadShared>(ks, 16 * c0, k_lds, kStripTiles, wave, lane_off, a.pitch);
+        stage_direct<C, kStripTiles, kReadShared>(vs, 16 * c0, v_lds, kStripTiles, wave, lane_off, a.pitch);
+        wait_direct();
+        __syncthreads();
+        if (c0 == 0) {
+            RowOperand<C> oop;
+            read_rows<C>(qop, q_lds + wave * LL::kTileBytes, row_lane);
+            read_rows<C>(gop, g_lds + wave * LL::kTileBytes, row_lane);
+            read_rows<C>(oop, o_lds + wave * LL::kTileBytes, row_lane);
+            dl = xor_sum(dot_lane<DT, C>(gop, oop));        // lane (n, g) holds a quarter of row n's channels
+        }
+        const int nk = min(kStripTiles, tiles - c0);
+#pragma unroll
+        for (int kt = 0; kt < kStripTiles; ++kt) {
+            if (kt >= nk) continue;
+            RowOperand<C> kop, vop;
+            read_rows<C>(kop, k_lds + kt * LL::kTileBytes, row_lane);
+            read_rows<C>(vop, v_lds + kt * LL::kTileBytes, row_lane);
+            const f32x4 s = dot_rows_mma<DT, C>(kop, qop);
+            const f32x4 dp = dot_rows_mma<DT, C>(vop, gop);
+            float dsv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = 16 * (c0 + kt) + 4 * g + r;
+                const float z = s[r] * scale2 - lse2 + ((key >= tv || row_masked) ? mask2 : 0.f);
+                const float p = key < T ? __builtin_amdgcn_exp2f(z) : 0.f;
+                dsv[r] = p * (dp[r] - dl);
+            }
+            const u32x2 db = {Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
+            LDS_PTR(char) blk = k_lds + kt * LL::kTileBytes;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(blk + tr_lane.off[ct]), db, acc[ct]);
+        }
+    }
+    if (qt >= tiles) return;
+    u32x2 qw[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[ct], a.scale);
+    store_tile<C>(dqs, qrow * a.pitch, qw, g, stores_whole_lines(a.pitch, C, 0), a.pitch);
+    if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(dl), ds, qrow * 4, 0, 0);
+}
+
+// =============================================================================
+// Backward, key side: dK and dV
+// =============================================================================
+template <class DT, int C>
+__global__ void __launch_bounds__(kThreads)
+global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__restrict__ q, const char *__restrict__ k,
+                  const char *__restrict__ v, const char *__restrict__ dout, const float *__restrict__ lse,
+                  const float *__restrict__ delta, const int32_t *__restrict__ t_valid, uint32_t items, GlobalArgs a) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16;
+    constexpr int kStep = region_bytes<C>(kStripTiles);
+    constexpr int kRows = 16 * kStripTiles;                 // rows of a chunk: one lse / delta value each
+    fetch_args_now(dk, dv, q, k, v, dout, lse, delta, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic,
+                   a.pitch, a.scale);
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 4 * kStep + 2 * kRows * 4 bytes
+    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) v_lds = k_lds + kStep;
+    LDS_PTR(char) q_lds = v_lds + kStep;
+    LDS_PTR(char) g_lds = q_lds + kStep;                    // dO
+    LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + kStep);
+    LDS_PTR(float) del_lds = lse_lds + kRows;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, n = lane & 15;
+    const uint32_t item = xcd_item(blockIdx.x, items);
+    const uint32_t b = div_by(item, a.strips, a.strips_magic);
+    const int strip = (int)(item - b * a.strips);
+    const uint32_t sample = div_by(b, a.H, a.heads_magic);
+    const int T = a.T, tiles = (T + 15) >> 4;
+    const int kt_own = kStripTiles * strip + wave;          // this wave's key tile
+    const int key = 16 * kt_own + n;
+
+    const int64_t seq_off = (int64_t)b * T * a.pitch;
+    const Rsrc qs = make_rsrc(q + seq_off, T * a.pitch), ks = make_rsrc(k + seq_off, T * a.pitch);
+    const Rsrc vs = make_rsrc(v + seq_off, T * a.pitch), gs = make_rsrc(dout + seq_off, T * a.pitch);
+    const Rsrc dks = make_rsrc(dk + seq_off, T * a.pitch), dvs = make_rsrc(dv + seq_off, T * a.pitch);
+    const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4), ds = make_rsrc(delta + (int64_t)b * T, T * 4);
+    const int lane_off = direct_lane_offset<C>(wave, lane, a.pitch, a.pitch);
+    int tv = T;
+    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
+    const bool col_masked = key >= tv;
+
+    RowLane<C> row_lane;
+    TrLane<C> tr_lane;
+    row_lane.init(0, lane);
+    tr_lane.init(0, lane);
+
+    const int row0 = 16 * kStripTiles * strip;
+    stage_direct<C, kStripTiles, kReadShared>(ks, row0, k_lds, kStripTiles, wave, lane_off, a.pitch);
+    stage_direct<C, kStripTiles, kReadShared>(vs, row0, v_lds, kStripTiles, wave, lane_off, a.pitch);
+    f32x4 acck[CT], accv[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) acck[ct] = accv[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    RowOperand<C> kop, vop;
+
+    for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
+        if (c0) __syncthreads();
+        stage_direct<C, kStripTiles, kReadShared>(qs, 16 * c0, q_lds, kStripTiles, wave, lane_off, a.pitch);
+        stage_direct<C, kStripTiles, kReadShared>(gs, 16 * c0, g_lds, kStripTiles, wave, lane_off, a.pitch);
+        if (wave == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))lse_lds, 4, (16 * c0 + lane) * 4, 0, 0, 0);
+        if (wave == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(ds, (LDS_PTR(void))del_lds, 4, (16 * c0 + lane) * 4, 0, 0, 0);
+        wait_direct();
+        __syncthreads();
+        if (c0 == 0) {
+            read_rows<C>(kop, k_lds + wave * LL::kTileBytes, row_lane);
+            read_rows<C>(vop, v_lds + wave * LL::kTileBytes, row_lane);
+        }
+        const int nq = min(kStripTiles, tiles - c0);        // query tiles in this chunk
+#pragma unroll
+        for (int qi = 0; qi < kStripTiles; ++qi) {
+            if (qi >= nq) continue;
+            RowOperand<C> qop, gop;
+            read_rows<C>(qop, q_lds + qi * LL::kTileBytes, row_lane);
+            read_rows<C>(gop, g_lds + qi * LL::kTileBytes, row_lane);
+            const f32x4 s = dot_rows_mma<DT, C>(qop, kop);   // [query 4g+r][key n]
+            const f32x4 dp = dot_rows_mma<DT, C>(gop, vop);
+            float p[4], dsv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int qloc = qi * 16 + 4 * g + r, qrow = 16 * c0 + qloc;
+                const float z = s[r] * scale2 - lse_lds[qloc] * kLog2e + ((col_masked || qrow >= tv) ? mask2 : 0.f);
+                p[r] = qrow < T ? __builtin_amdgcn_exp2f(z) : 0.f;     // rows past the sequence do not exist
+                dsv[r] = p[r] * (dp[r] - del_lds[qloc]);
+            }
+            const u32x2 pb = {Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+            const u32x2 db = {Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
+            LDS_PTR(char) qtile = q_lds + qi * LL::kTileBytes;
+            LDS_PTR(char) gtile = g_lds + qi * LL::kTileBytes;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                accv[ct] = Mma<DT>::k16(read_tr(gtile + tr_lane.off[ct]), pb, accv[ct]);
+                acck[ct] = Mma<DT>::k16(read_tr(qtile + tr_lane.off[ct]), db, acck[ct]);
+            }
+        }
+    }
+    if (kt_own >= tiles) return;
+    u32x2 kw[CT], vw[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        kw[ct] = pack_acc<DT>(acck[ct], a.scale);
+        vw[ct] = pack_acc<DT>(accv[ct], 1.f);
+    }
+    const bool stream = stores_whole_lines(a.pitch, C, 0);
+    store_tile<C>(dks, key * a.pitch, kw, g, stream, a.pitch);      // rows past T are dropped
+    store_tile<C>(dvs, key * a.pitch, vw, g, stream, a.pitch);
+}
+
+// ----------------------------------------------------------------------------- launchers
+template <int C> constexpr size_t global_lds(int regions) {
+    return (size_t)regions * region_bytes<C>(kStripTiles) + 2 * 16 * kStripTiles * sizeof(float);
+}
+inline bool global_ok(const Geom &g, GlobalArgs &a, int64_t &items) {
+    if (g.C > 128 || g.T > (1 << 28) / g.C) return false;
+    const int tiles = (int)((g.T + 15) / 16);
+    a.T = (int)g.T;
+    a.H = g.H;
+    a.strips = (tiles + kStripTiles - 1) / kStripTiles;
+    items = g.B * a.strips;
+    if (items > 0x7fffff00LL || !div_magic_ok(items, a.strips) || !div_magic_ok(g.B, g.H)) return false;
+    a.strips_magic = div_magic(a.strips);
+    a.heads_magic = div_magic(g.H);
+    a.pitch = 2 * g.C;
+    return true;
+}
+
+template <class DT, int C>
+int launch_global_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
+                      const Geom &g, float scale, hipStream_t s) {
+    GlobalArgs a;
+    int64_t items;
+    if (!global_ok(g, a, items)) return NA1D_ERR_UNSUPPORTED;
+    a.scale = scale;
+    if (!allow_lds(global_fwd_kernel<DT, C>, global_lds<C>(3))) return NA1D_ERR_LAUNCH;
+    global_fwd_kernel<DT, C><<<(unsigned)items, kThreads, global_lds<C>(3), s>>>((char *)out, lse, (const char *)q, (const char *)k,
+                                                                 (const char *)v, t_valid, (uint32_t)items, a);
+    return launch_status();
+}
+
+template <class DT, int C>
+int launch_global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q, const void *k, const void *v,
+                      const void *out, const void *dout, const float *lse, const int32_t *t_valid, const Geom &g,
+                      float scale, hipStream_t s) {
+    GlobalArgs a;
+    int64_t items;
+    if (!global_ok(g, a, items)) return NA1D_ERR_UNSUPPORTED;
+    a.scale = scale;
+    if (!allow_lds(global_dq_kernel<DT, C>, global_lds<C>(5)) || !allow_lds(global_dkv_kernel<DT, C>, global_lds<C>(4)))
+        return NA1D_ERR_LAUNCH;
+    global_dq_kernel<DT, C><<<(unsigned)items, kThreads, global_lds<C>(5), s>>>((char *)dq, delta, (const char *)q, (const char *)k,
+                                                                (const char *)v, (const char *)out, (const char *)dout,
+                                                                lse, t_valid, (uint32_t)items, a);
+    global_dkv_kernel<DT, C><<<(unsigned)items, kThreads, global_lds<C>(4), s>>>((char *)dk, (char *)dv, (const char *)q, (const char *)k,
+                                                                 (const char *)v, (const char *)dout, lse, delta, t_valid,
+                                                                 (uint32_t)items, a);
+    return launch_status();
+}
+
+int global_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
+               const Geom &g, float scale, int dtype, hipStream_t s) {
+    NA1D_MFMA_DISPATCH(launch_global_fwd, out, lse, q, k, v, t_valid, g, scale, s);
+}
+
+int global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q, const void *k, const void *v, const void *out,
+               const void *dout, const float *lse, const int32_t *t_valid, const Geom &g, float scale, int dtype,
+               hipStream_t s) {
+    NA1D_MFMA_DISPATCH(launch_global_bwd, dq, dk, dv, delta, q, k, v, out, dout, lse, t_valid, g, scale, s);
+}
+
+}  // namespace mfma
+}  // namespace na1d

@@ -22,6 +22,7 @@ _UNFUSED = ("na1d_qk_forward", "na1d_av_forward", "na1d_q_backward", "na1d_k_bac
             "na1d_a_backward", "na1d_v_backward")
 SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_backward_workspace_bytes",
                       "na1d_fused_forward_strided", "na1d_fused_backward_strided", "na1d_profile_events",
+                      "na1d_global_forward", "na1d_global_backward", "na1d_global_backward_workspace_bytes",
                       "na1d_version", "na1d_status_string")
 UNSUPPORTED = -8
 
@@ -60,6 +61,12 @@ def load():
     lib.na1d_fused_backward_strided.argtypes = [_ptr] * 11 + [_i64] * 6 + [_f32, _int, _ptr, _ptr, _ptr, _i64, _ptr]
     lib.na1d_fused_backward_workspace_bytes.restype = _i64
     lib.na1d_fused_backward_workspace_bytes.argtypes = [_i64] * 6 + [_int]
+    lib.na1d_global_forward.restype = _int
+    lib.na1d_global_forward.argtypes = [_ptr] * 6 + [_i64] * 4 + [_f32, _int, _ptr]
+    lib.na1d_global_backward.restype = _int
+    lib.na1d_global_backward.argtypes = [_ptr] * 10 + [_i64] * 4 + [_f32, _int, _ptr, _i64, _ptr]
+    lib.na1d_global_backward_workspace_bytes.restype = _i64
+    lib.na1d_global_backward_workspace_bytes.argtypes = [_i64] * 4 + [_int]
     lib.na1d_profile_events.restype = _int
     lib.na1d_profile_events.argtypes = [_ptr, _ptr]
     lib.na1d_version.restype = _int
@@ -160,3 +167,30 @@ def call_fused_backward_strided(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_val
     if st != UNSUPPORTED:
         check(st, "na1d_fused_backward_strided")
     return st
+
+
+def call_global_forward(out, lse, q, k, v, t_valid, B, H, T, C, scale):
+    """Dense attention over whole sequences; returns the status (``UNSUPPORTED`` for head_dim > 128)."""
+    lib = load()
+    with torch.cuda.device(out.device):
+        st = lib.na1d_global_forward(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(t_valid), B, H, T, C, scale,
+                                     dtype_tag(q.dtype), _stream(out))
+    if st != UNSUPPORTED:
+        check(st, "na1d_global_forward")
+    return st
+
+
+def global_backward_workspace_bytes(B, H, T, C, dtype) -> int:
+    n = load().na1d_global_backward_workspace_bytes(B, H, T, C, dtype_tag(dtype))
+    if n < 0:
+        check(int(n), "na1d_global_backward_workspace_bytes")
+    return int(n)
+
+
+def call_global_backward(dq, dk, dv, q, k, v, out, dout, lse, t_valid, B, H, T, C, scale, workspace):
+    lib = load()
+    with torch.cuda.device(dq.device):
+        st = lib.na1d_global_backward(_p(dq), _p(dk), _p(dv), _p(q), _p(k), _p(v), _p(out), _p(dout), _p(lse),
+                                      _p(t_valid), B, H, T, C, scale, dtype_tag(q.dtype), _p(workspace),
+                                      workspace.numel() * workspace.element_size(), _stream(dq))
+    check(st, "na1d_global_backward")

@@ -28,6 +28,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from .dense import global_attention
 from .fused import na1d_fused, na1d_fused_qkv
 from .nattn import getNA1dFunction
 
@@ -331,19 +332,28 @@ class NAttention(nn.Module):
 class GlobalAttention(nn.Module):
     """Dense attention with an additive sinusoid input (PCF :181-225 / MFA :180-221)."""
 
-    def __init__(self, dim, num_heads, groups=1, channels_first=True):
+    def __init__(self, dim, num_heads, groups=1, channels_first=True, dense="native"):
         super().__init__()
-        self.num_heads, self.groups, self.channels_first = num_heads, groups, channels_first
+        assert dense in ("native", "sdpa")
+        self.num_heads, self.groups, self.channels_first, self.dense = num_heads, groups, channels_first, dense
         self.scale = (dim // num_heads) ** -0.5
         self.linear_pos = _Projection.make(dim, dim, False, groups, channels_first)
         self.qkv = _Projection.make(dim, dim * 3, True, groups, channels_first)
         self.proj = _Projection.make(dim, dim, True, groups, channels_first)
 
-    def forward(self, x, pos_emb, attn_mask=None):
+    def forward(self, x, pos_emb, attn_mask=None, padding=None):
+        """``padding`` [N] (patches) says the same as ``attn_mask`` (-100 on padded rows and columns); the HIP
+        kernels build the mask from it, the other paths add the tensor."""
         n = x.shape[0]
         x = x + self.linear_pos(pos_emb.to(x.dtype))
         q, k, v = _split_heads(self.qkv(x), self.num_heads, self.groups, self.channels_first)
         t, hd = q.shape[1], q.shape[2]
+        native = (self.dense == "native" and x.device.type == "cuda" and hd <= 128 and hd % 8 == 0
+                  and q.dtype in (torch.bfloat16, torch.float16) and (attn_mask is None or padding is not None))
+        if native:                       # the HIP kernels: no mask or score tensor
+            t_valid = None if attn_mask is None else (t - padding).clamp(0, t).to(torch.int32)
+            out = global_attention(q.contiguous(), k.contiguous(), v.contiguous(), self.num_heads, t_valid, self.scale)
+            return self.proj(_merge_heads(out, n, self.num_heads, self.channels_first))
         q, k, v = (z.view(n, self.num_heads, t, hd) for z in (q, k, v))
         if x.device.type == "cuda":      # one library kernel instead of matmul -> mask -> softmax -> matmul
             out = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, scale=self.scale)
@@ -386,7 +396,11 @@ class NATFLayer(nn.Module):
 
     def forward(self, x, padding=None, pos_emb=None, attn_mask_global=None):
         y = self.norm1(x)
-        y = self.attn(y, padding=padding) if self.local else self.attn(y, pos_emb=pos_emb, attn_mask=attn_mask_global)
+        if self.local:
+            y = self.attn(y, padding=padding)
+        else:
+            y = self.attn(y, pos_emb=pos_emb, attn_mask=attn_mask_global,
+                          padding=padding if attn_mask_global is not None else None)
         x = x + self.drop_path(y)
         return x + self.drop_path(self.mlp(self.norm2(x)))
 

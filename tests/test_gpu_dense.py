@@ -1,0 +1,85 @@
+"""GPU parity of the dense ("global") attention kernels against the CPU oracle, through the C ABI."""
+import pytest
+import torch
+
+from oracle import na1d_oracle as O
+from na1d_amd import _lib
+from na1d_amd.dense import global_attention
+from _util import TOL, make_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+DTYPES = [torch.bfloat16, torch.float16]
+GEOMS = [  # (N, H, T, C): one tile, ragged tiles, several strips and chunks, every kernel width, padded widths
+    (1, 1, 1, 16), (2, 2, 16, 16), (3, 2, 37, 32), (2, 4, 64, 16), (3, 1, 65, 64), (2, 2, 130, 32), (1, 2, 300, 16),
+    (2, 1, 129, 128), (2, 2, 100, 24), (1, 3, 77, 48), (2, 1, 90, 104), (1, 1, 1000, 32),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_global_attention_matches_oracle(geom, dtype):
+    N, H, T, C = geom
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, 0, 77, dtype, n=4)
+    scale = C ** -0.5
+    pad = torch.tensor([0, T // 2, T][:N])
+    t_valid = (T - pad).to(torch.int32)
+    print("global attention", geom, dtype, flush=True)
+
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = global_attention(qd, kd, vd, H, t_valid=t_valid.cuda(), scale=scale)
+    out.backward(do.cuda())
+    torch.cuda.synchronize()
+
+    qf, kf, vf = q.float(), k.float(), v.float()
+    want_o, _, want_lse = O.global_forward(qf, kf, vf, scale, pad, H)
+    wq, wk, wv = O.global_backward(qf, kf, vf, do.float(), scale, pad, H)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float(), want_o) < tol, "O"
+    assert O.rel_l2(qd.grad.float(), wq) < tol, "dQ"
+    assert O.rel_l2(kd.grad.float(), wk) < tol, "dK"
+    assert O.rel_l2(vd.grad.float(), wv) < tol, "dV"
+    lse = torch.empty(B, T, dtype=torch.float32, device="cuda")
+    o2 = torch.empty_like(qd)
+    assert _lib.call_global_forward(o2, lse, qd.detach(), kd.detach(), vd.detach(), t_valid.cuda(), B, H, T, C, scale) == 0
+    assert torch.allclose(lse.cpu(), want_lse, atol=2e-3, rtol=1e-4), "LSE"
+    assert torch.equal(o2, out)
+
+
+def test_global_attention_without_padding_and_without_lse():
+    N, H, T, C, dtype = 2, 2, 150, 32, torch.bfloat16
+    B = N * H
+    q, k, v = make_inputs(B, T, C, 0, 5, dtype)
+    qd, kd, vd = (t.cuda() for t in (q, k, v))
+    out = torch.empty_like(qd)
+    assert _lib.call_global_forward(out, None, qd, kd, vd, None, B, H, T, C, 0.2) == 0
+    want, _, _ = O.global_forward(q.float(), k.float(), v.float(), 0.2, None, H)
+    assert O.rel_l2(out.float(), want) < TOL[dtype]
+
+
+def test_global_attention_is_deterministic_and_leaves_neighbours_alone():
+    """Every output is written once by one wave: two runs agree bit for bit, and rows of neighbouring
+    sequences (T not a multiple of the tile) are not touched by the ragged last tile."""
+    N, H, T, C, dtype = 2, 3, 41, 32, torch.float16
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, 0, 9, dtype, n=4)
+    grads = []
+    for _ in range(2):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        global_attention(qd, kd, vd, H).backward(do.cuda())
+        grads.append((qd.grad, kd.grad, vd.grad))
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+    # sequence b alone equals sequence b inside the batch
+    qd, kd, vd = (t[2:3].contiguous().cuda() for t in (q, k, v))
+    alone = global_attention(qd, kd, vd, 1)
+    full = global_attention(q.cuda(), k.cuda(), v.cuda(), H)
+    assert torch.equal(alone[0], full[2])
+
+
+def test_global_attention_rejects_wide_heads():
+    q = torch.zeros(1, 4, 136, dtype=torch.bfloat16, device="cuda")
+    out = torch.empty_like(q)
+    assert _lib.call_global_forward(out, None, q, q, q, None, 1, 1, 4, 136, 1.0) == _lib.UNSUPPORTED

@@ -8,6 +8,7 @@ import math
 
 import pytest
 import torch
+import torch.nn.functional as F
 
 from oracle import na1d_oracle as O
 
@@ -259,3 +260,71 @@ def test_seeded_inputs_are_reproducible_and_rounded():
     assert all(torch.equal(x, y) for x, y in zip(a, b))
     assert a[0].dtype == torch.bfloat16
     assert math.isclose(O.rel_l2(a[1].float(), a[1].float()), 0.0)
+
+
+# --------------------------------------------------------------------------
+# dense attention of the global layers
+# --------------------------------------------------------------------------
+def test_global_mask_closed_form():
+    T, pads = 7, [0, 3, 7]
+    m = O.global_mask(T, pads)
+    assert m.shape == (3, T, T)
+    for n, pad in enumerate(pads):
+        for t in range(T):
+            for u in range(T):
+                want = O.MASK_VALUE if (t >= T - pad or u >= T - pad) else 0.0
+                assert m[n, t, u].item() == want
+    assert O.global_mask(T).abs().sum() == 0
+
+
+def test_global_forward_matches_index_loops():
+    import math
+    N, H, T, C, scale, pads = 2, 2, 5, 3, 0.37, [0, 2]
+    q, k, v = _rand(N * H, T, C), _rand(N * H, T, C), _rand(N * H, T, C)
+    o, p, lse = O.global_forward(q, k, v, scale, pads, H)
+    for b in range(N * H):
+        tv = T - pads[b // H]
+        for t in range(T):
+            z = [sum(q[b, t, c].item() * k[b, u, c].item() for c in range(C)) * scale
+                 + (O.MASK_VALUE if (t >= tv or u >= tv) else 0.0) for u in range(T)]
+            den = sum(math.exp(x) for x in z)
+            assert abs(lse[b, t].item() - math.log(den)) < 1e-9
+            for c in range(C):
+                want = sum(math.exp(z[u]) / den * v[b, u, c].item() for u in range(T))
+                assert abs(o[b, t, c].item() - want) < 1e-9
+
+
+def test_global_forward_matches_library_attention():
+    N, H, T, C, scale, pads = 2, 3, 11, 8, 0.2, [4, 0]
+    q, k, v = _rand(N * H, T, C), _rand(N * H, T, C), _rand(N * H, T, C)
+    o, _, _ = O.global_forward(q, k, v, scale, pads, H)
+    m = O.global_mask(T, pads, dtype=q.dtype).unsqueeze(1)
+    want = F.scaled_dot_product_attention(q.view(N, H, T, C), k.view(N, H, T, C), v.view(N, H, T, C), attn_mask=m,
+                                          scale=scale)
+    assert torch.allclose(o.view(N, H, T, C), want, atol=1e-10)
+
+
+def test_global_forward_equals_full_window_na1d():
+    # a window that reaches every key from every row, no bias, no padding: the out-of-range slots carry -100 and
+    # zero keys, i.e. weights of e^-100 relative to the in-range ones
+    B, T, C = 2, 6, 4
+    q, k, v = _rand(B, T, C), _rand(B, T, C), _rand(B, T, C)
+    o_dense, _, lse_dense = O.global_forward(q, k, v, 1.0)
+    o_band, _, lse_band = O.na1d_forward(q, k, v, 2 * T - 1, T - 1)
+    assert torch.allclose(o_dense, o_band, atol=1e-12)
+    assert torch.allclose(lse_dense, lse_band, atol=1e-12)
+
+
+def test_global_gradcheck_fp64():
+    N, H, T, C = 2, 2, 5, 3
+    q, k, v = (_rand(N * H, T, C).requires_grad_(True) for _ in range(3))
+    assert torch.autograd.gradcheck(lambda a, b, c: O.global_forward(a, b, c, 0.4, [1, 0], H)[0], (q, k, v), atol=1e-7)
+    do = _rand(N * H, T, C)
+    dq, dk, dv = O.global_backward(q, k, v, do, 0.4, [1, 0], H)
+    # the textbook softmax-attention gradients
+    o, p, _ = O.global_forward(q.detach(), k.detach(), v.detach(), 0.4, [1, 0], H)
+    dp = torch.einsum("btc,buc->btu", do, v.detach())
+    ds = p * (dp - (do * o).sum(-1, keepdim=True))
+    assert torch.allclose(dv, torch.einsum("btu,btc->buc", p, do), atol=1e-12)
+    assert torch.allclose(dq, 0.4 * torch.einsum("btu,buc->btc", ds, k.detach()), atol=1e-12)
+    assert torch.allclose(dk, 0.4 * torch.einsum("btu,btc->buc", ds, q.detach()), atol=1e-12)
