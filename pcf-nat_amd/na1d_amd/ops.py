@@ -209,3 +209,72 @@ def na1d_fused_op(q: Tensor, k: Tensor, v: Tensor, win_size: int, left: int, rpb
     ``[num_heads, win_size]`` fp32 (reshape the model's ``[1, H, 1, W]`` parameter), ``t_valid`` int32 ``[N]``."""
     return getattr(torch.ops, NAMESPACE).na1d_fused_forward(q, k, v, rpb, t_valid, num_heads, win_size, left,
                                                             float(scale))[0]
+
+
+# --------------------------------------------------------------------------- dense attention of the global layers
+_library.define("global_attention_forward(Tensor q, Tensor k, Tensor v, Tensor? t_valid, int num_heads, float scale) "
+                "-> (Tensor, Tensor)")
+_library.define("global_attention_backward(Tensor dout, Tensor q, Tensor k, Tensor v, Tensor out, Tensor lse, "
+                "Tensor? t_valid, int num_heads, float scale) -> (Tensor, Tensor, Tensor)")
+
+
+def _dense_forward(q, k, v, t_valid, num_heads, scale):
+    _fused_contract(q, k, v, None, t_valid, num_heads, 0)
+    B, T, C = q.shape
+    out = torch.empty_like(q)
+    lse = torch.empty((B, T), dtype=torch.float32, device=q.device)
+    torch._check(_lib.call_global_forward(out, lse, q, k, v, t_valid, B, num_heads, T, C, scale) == 0,
+                 lambda: "dense attention covers head_dim <= 128")
+    return out, lse
+
+
+def _dense_forward_fake(q, k, v, t_valid, num_heads, scale):
+    _fused_contract(q, k, v, None, t_valid, num_heads, 0)
+    return torch.empty_like(q), torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
+
+
+def _dense_backward(dout, q, k, v, out, lse, t_valid, num_heads, scale):
+    B, T, C = q.shape
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    if B * T:
+        ws = torch.empty(_lib.global_backward_workspace_bytes(B, num_heads, T, C, q.dtype), dtype=torch.uint8,
+                         device=q.device)
+        _lib.call_global_backward(dq, dk, dv, q, k, v, out, dout.contiguous(), lse, t_valid, B, num_heads, T, C, scale,
+                                  ws)
+    return dq, dk, dv
+
+
+def _dense_backward_fake(dout, q, k, v, out, lse, t_valid, num_heads, scale):
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+
+_library.impl("global_attention_forward", _dense_forward, "CUDA")
+_library.impl("global_attention_backward", _dense_backward, "CUDA")
+torch.library.register_fake(NAMESPACE + "::global_attention_forward", _dense_forward_fake, lib=_library)
+torch.library.register_fake(NAMESPACE + "::global_attention_backward", _dense_backward_fake, lib=_library)
+
+
+def _dense_setup(ctx, inputs, output):
+    q, k, v, t_valid, ctx.num_heads, ctx.scale = inputs
+    out, lse = output
+    ctx.has_tv = t_valid is not None
+    ctx.save_for_backward(*[t for t in (q, k, v, out, lse, t_valid) if t is not None])
+
+
+def _dense_autograd(ctx, dout, _dlse):
+    saved = list(ctx.saved_tensors)
+    q, k, v, out, lse = saved[:5]
+    t_valid = saved[5] if ctx.has_tv else None
+    dq, dk, dv = getattr(torch.ops, NAMESPACE).global_attention_backward(dout, q, k, v, out, lse, t_valid,
+                                                                         ctx.num_heads, ctx.scale)
+    return dq, dk, dv, None, None, None
+
+
+torch.library.register_autograd(NAMESPACE + "::global_attention_forward", _dense_autograd, setup_context=_dense_setup,
+                                lib=_library)
+
+
+def global_attention_op(q: Tensor, k: Tensor, v: Tensor, num_heads: int = 1, t_valid: Optional[Tensor] = None,
+                        scale: float = 1.0) -> Tensor:
+    """:func:`na1d_amd.dense.global_attention` through the registered op (traceable by ``torch.compile``)."""
+    return getattr(torch.ops, NAMESPACE).global_attention_forward(q, k, v, t_valid, num_heads, float(scale))[0]

@@ -70,3 +70,27 @@ def test_compiled_function_through_the_ops_matches_eager_and_the_oracle(dtype):
     assert O.rel_l2(fc.float(), want) < TOL[dtype]
     ref = na1d_fused(ins_e[0].detach(), ins_e[1].detach(), ins_e[2].detach(), W, L, rpb=rpb.cuda(), t_valid=tv, num_heads=H)
     assert torch.equal(fc, ref)
+
+
+def test_dense_attention_op_compiles_and_equals_the_eager_operator():
+    from na1d_amd.dense import global_attention
+    N, H, T, C, dtype = 2, 2, 70, 32, torch.bfloat16
+    q, k, v, do = make_inputs(N * H, T, C, 0, 21, dtype, n=4)
+    pad = torch.tensor([0, 30])
+    tv = (T - pad).to(torch.int32).cuda()
+    fn = lambda q, k, v: ops.global_attention_op(q, k, v, H, tv, C ** -0.5)
+    compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    ins_c = [t.cuda().requires_grad_(True) for t in (q, k, v)]
+    ins_e = [t.cuda().requires_grad_(True) for t in (q, k, v)]
+    oc = compiled(*ins_c)
+    oc.backward(do.cuda())
+    oe = global_attention(*ins_e, H, tv, C ** -0.5)
+    oe.backward(do.cuda())
+    assert torch.equal(oc, oe)
+    for x, y in zip(ins_c, ins_e):
+        assert torch.equal(x.grad, y.grad)
+    want, _, _ = O.global_forward(q.float(), k.float(), v.float(), C ** -0.5, pad, H)
+    assert O.rel_l2(oc.float(), want) < TOL[dtype]
+    x = q.cuda()
+    torch.library.opcheck(torch.ops.na_cuda.global_attention_forward.default, (x, x, x, tv, H, 0.2),
+                          test_utils=["test_schema", "test_faketensor"])

@@ -37,6 +37,9 @@ def test_fake_kernels_propagate_shapes(prefix, dtype):
         getattr(ns, prefix + "_ana_av_forward")(s, x, N, T, C, W + 1, L)                 # score tensor of another window
     o, lse = ns.na1d_fused_forward(x, x, x, None, None, 1, W, L, 1.0)
     assert o.shape == (N, T, C) and lse.shape == (N, T) and lse.dtype == torch.float32
+    o, lse = ns.global_attention_forward(x, x, x, None, 1, 1.0)
+    assert o.shape == (N, T, C) and o.dtype == dtype and lse.shape == (N, T) and lse.dtype == torch.float32
+    assert all(g.shape == (N, T, C) for g in ns.global_attention_backward(x, x, x, x, x, lse, None, 1, 1.0))
 
 
 def test_wrappers_pick_the_op_by_dtype():
