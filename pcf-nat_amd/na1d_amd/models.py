@@ -265,8 +265,9 @@ class NAttention(nn.Module):
     """Neighbourhood attention layer (PCF_NATransformer.py:44-178 / MFA_NATransformer.py:43-177)."""
 
     def __init__(self, frames, dim, num_heads, win_size, groups=1, channels_first=True, dtype=torch.bfloat16,
-                 na="fused", dilation=1):
+                 na="fused", dilation=1, attn_drop=0.0, proj_drop=0.0):
         super().__init__()
+        self.attn_drop, self.proj_drop = attn_drop, nn.Dropout(proj_drop)      # PCF :71-73
         if isinstance(win_size, int):
             assert win_size > 0
             left = win_size - 1 - win_size // 2
@@ -283,7 +284,10 @@ class NAttention(nn.Module):
         nn.init.normal_(self.relative_position_bias, mean=0.0, std=0.02)
         self.proj = _Projection.make(dim, dim, True, groups, channels_first)
         self.register_buffer("attn_mask", _window_mask(frames, win_size, left, None, torch.float32, "cpu").unsqueeze(1))
-        if na == "unfused":     # like the reference's CUDA path, the two-call chain has no dilated kernels
+        # The fused kernels never hold the probabilities in memory, so attention dropout (PCF :149; 0 in every
+        # configuration of the reference) is applied where the reference applies it: in the two-call chain.
+        self._chain = na == "unfused" or attn_drop > 0.0
+        if self._chain:         # like the reference's CUDA path, the two-call chain has no dilated kernels
             self.NA1d_QK_Function, self.NA1d_AV_Function = getNA1dFunction(C=head_dim, dilation=dilation, dtype=dtype)
 
     def forward(self, x, padding=None):
@@ -291,22 +295,24 @@ class NAttention(nn.Module):
         t = x.shape[-1] if self.channels_first else x.shape[1]
         h, w, left = self.num_heads, self.win_size, self.left
         t_valid = None if padding is None else (t - padding).to(torch.int32)
-        if self.na == "fused_qkv":
-            return self._forward_token_major(x, n, t, t_valid)
+        dropping = self.attn_drop > 0.0 and self.training
+        if self.na == "fused_qkv" and not dropping:
+            return self.proj_drop(self._forward_token_major(x, n, t, t_valid))
         q, k, v = _split_heads(self.qkv(x), h, self.groups, self.channels_first)
         q = q * self.scale                                   # in the activation dtype, as the reference does (:141)
         extra = {} if self.dilation == 1 else {"dilation": self.dilation}
         if callable(self.na):
             out = self.na(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h, **extra)
-        elif self.na == "fused":
+        elif self.na in ("fused", "fused_qkv") and not dropping:
             out = na1d_fused(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h, **extra)
         else:                                                # the reference's un-fused chain (:141-150)
             attn = self.NA1d_QK_Function.apply(q, k, w, left, 1).view(n, h, t, w)
             attn = attn + self.relative_position_bias
             attn = attn + _window_mask(t, w, left, padding, x.dtype, x.device).unsqueeze(1)
             attn = torch.softmax(attn.view(n * h, t, w), dim=-1)
+            attn = F.dropout(attn, self.attn_drop, self.training)
             out = self.NA1d_AV_Function.apply(attn, v, w, left, 1)
-        return self.proj(_merge_heads(out, n, h, self.channels_first))
+        return self.proj_drop(self.proj(_merge_heads(out, n, h, self.channels_first)))
 
     def _forward_token_major(self, x, n, t, t_valid):
         """The same layer with the operator reading the qkv projection in place.  Tokens-first models have the
@@ -332,10 +338,11 @@ class NAttention(nn.Module):
 class GlobalAttention(nn.Module):
     """Dense attention with an additive sinusoid input (PCF :181-225 / MFA :180-221)."""
 
-    def __init__(self, dim, num_heads, groups=1, channels_first=True, dense="native"):
+    def __init__(self, dim, num_heads, groups=1, channels_first=True, dense="native", attn_drop=0.0, proj_drop=0.0):
         super().__init__()
         assert dense in ("native", "sdpa")
         self.num_heads, self.groups, self.channels_first, self.dense = num_heads, groups, channels_first, dense
+        self.attn_drop, self.proj_drop = attn_drop, nn.Dropout(proj_drop)      # PCF :193-195
         self.scale = (dim // num_heads) ** -0.5
         self.linear_pos = _Projection.make(dim, dim, False, groups, channels_first)
         self.qkv = _Projection.make(dim, dim * 3, True, groups, channels_first)
@@ -348,50 +355,54 @@ class GlobalAttention(nn.Module):
         x = x + self.linear_pos(pos_emb.to(x.dtype))
         q, k, v = _split_heads(self.qkv(x), self.num_heads, self.groups, self.channels_first)
         t, hd = q.shape[1], q.shape[2]
-        native = (self.dense == "native" and x.device.type == "cuda" and hd <= 128 and hd % 8 == 0
+        drop_p = self.attn_drop if self.training else 0.0
+        native = (self.dense == "native" and x.device.type == "cuda" and hd <= 128 and hd % 8 == 0 and drop_p == 0.0
                   and q.dtype in (torch.bfloat16, torch.float16) and (attn_mask is None or padding is not None))
         if native:                       # the HIP kernels: no mask or score tensor
             t_valid = None if attn_mask is None else (t - padding).clamp(0, t).to(torch.int32)
             out = global_attention(q.contiguous(), k.contiguous(), v.contiguous(), self.num_heads, t_valid, self.scale)
-            return self.proj(_merge_heads(out, n, self.num_heads, self.channels_first))
+            return self.proj_drop(self.proj(_merge_heads(out, n, self.num_heads, self.channels_first)))
         q, k, v = (z.view(n, self.num_heads, t, hd) for z in (q, k, v))
         if x.device.type == "cuda":      # one library kernel instead of matmul -> mask -> softmax -> matmul
-            out = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, scale=self.scale)
+            out = F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, dropout_p=drop_p, scale=self.scale)
         else:
             attn = (q * self.scale) @ k.transpose(-2, -1)
             if attn_mask is not None:
                 attn = attn + attn_mask
-            out = torch.softmax(attn, dim=-1) @ v
-        return self.proj(_merge_heads(out.reshape(n * self.num_heads, t, hd), n, self.num_heads, self.channels_first))
+            out = F.dropout(torch.softmax(attn, dim=-1), drop_p) @ v
+        out = _merge_heads(out.reshape(n * self.num_heads, t, hd), n, self.num_heads, self.channels_first)
+        return self.proj_drop(self.proj(out))
 
 
 class Mlp(nn.Module):
-    def __init__(self, dim, hidden, groups, channels_first):
+    def __init__(self, dim, hidden, groups, channels_first, drop=0.0):
         super().__init__()
         self.fc1 = _Projection.make(dim, hidden, True, groups, channels_first)
         self.act = nn.GELU()
         self.fc2 = _Projection.make(hidden, dim, True, groups, channels_first)
+        self.drop = nn.Dropout(drop)                            # PCF :33-40
 
     def forward(self, x):
-        return self.fc2(self.act(self.fc1(x)))
+        return self.drop(self.fc2(self.drop(self.act(self.fc1(x)))))
 
 
 class NATFLayer(nn.Module):
     """norm -> attention -> residual; norm -> MLP -> residual (PCF :228-265)."""
 
     def __init__(self, frames, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na, mlp_ratio=4,
-                 dilation=1):
+                 dilation=1, attn_drop=0.0, drop=0.0):
         super().__init__()
         self.local = isinstance(win_size, list) or win_size > 0
         if self.local:
-            self.attn = NAttention(frames, dim, num_heads, win_size, groups, channels_first, dtype, na, dilation)
+            self.attn = NAttention(frames, dim, num_heads, win_size, groups, channels_first, dtype, na, dilation,
+                                   attn_drop, drop)
         else:
             assert dilation == 1
-            self.attn = GlobalAttention(dim, num_heads, groups, channels_first)
+            self.attn = GlobalAttention(dim, num_heads, groups, channels_first, attn_drop=attn_drop, proj_drop=drop)
         norm = BatchNorm1d if channels_first else TokenBatchNorm
         self.norm1 = norm(dim)
         self.drop_path = DropPath(drop_path) if drop_path > 0.0 else nn.Identity()
-        self.mlp = Mlp(dim, int(dim * mlp_ratio), groups, channels_first)
+        self.mlp = Mlp(dim, int(dim * mlp_ratio), groups, channels_first, drop)
         self.norm2 = norm(dim)
 
     def forward(self, x, padding=None, pos_emb=None, attn_mask_global=None):
@@ -407,13 +418,14 @@ class NATFLayer(nn.Module):
 
 class NATFBlock(nn.Module):
     def __init__(self, frames, depth, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na,
-                 use_checkpoint=False, dilation=1):
+                 use_checkpoint=False, dilation=1, attn_drop=0.0, drop=0.0):
         super().__init__()
         pick = lambda v, i: v[i] if isinstance(v, list) else v
         self.use_checkpoint = use_checkpoint if isinstance(use_checkpoint, list) else [use_checkpoint] * depth
         self.blocks = nn.ModuleList([
             NATFLayer(frames, dim, pick(num_heads, i), pick(win_size, i), pick(groups, i), pick(drop_path, i),
-                      channels_first, dtype, na, dilation=pick(dilation, i)) for i in range(depth)])
+                      channels_first, dtype, na, dilation=pick(dilation, i), attn_drop=attn_drop, drop=drop)
+            for i in range(depth)])
 
     def forward(self, x, padding=None, pos_emb=None, attn_mask_global=None):
         for layer, ckpt in zip(self.blocks, self.use_checkpoint):
@@ -441,7 +453,7 @@ class _NATransformer(nn.Module):
     def __init__(self, channels_first, frames=300, patch_size=2, in_chans=80, output_emb_size=192, embed_dim=256,
                  depths=(4, 4, 4, 4), num_heads=None, win_size=None, groups=(8, 4, 2, 1), drop_path_rate=0.0,
                  proj_channel=1536, asp=True, poolnorm=True, use_checkpoint=False, dtype=torch.bfloat16, na="fused",
-                 dilation=1):
+                 dilation=1, attn_drop=0.0, drop=0.0):
         super().__init__()
         depths = list(depths)
         nb = len(depths)
@@ -463,7 +475,8 @@ class _NATransformer(nn.Module):
         self.blocks = nn.ModuleList([
             NATFBlock(emb_frames, depths[i], embed_dim, pick(num_heads, i), pick(win_size, i),
                       pick(groups, i) if channels_first else 1, dpr[sum(depths[:i]):sum(depths[:i + 1])],
-                      channels_first, dtype, na, pick(use_checkpoint, i), pick(dilation, i)) for i in range(nb)])
+                      channels_first, dtype, na, pick(use_checkpoint, i), pick(dilation, i), attn_drop, drop)
+            for i in range(nb)])
         self.norm = BatchNorm1d(embed_dim * nb)
         self.proj = TDNNBlock(embed_dim * nb, proj_channel, 1)
         self.pool = AttentiveStatisticsPooling(proj_channel) if asp else StatisticsPooling()

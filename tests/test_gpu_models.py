@@ -136,3 +136,25 @@ def test_mfa_nat_4x4_training_step_fp16(na):
     scaler.step(opt)
     scaler.update()
     assert not torch.equal(before, gpu.fc.weight.detach())
+
+
+def test_attention_dropout_runs_through_the_two_call_chain():
+    """attn_drop / drop of the reference's constructors (models/PCF_NATransformer.py:324,375; 0 in its
+    configurations): inactive in eval mode, and in training the probabilities are dropped where the reference
+    drops them, between the two calls of the un-fused chain."""
+    kw = dict(depths=(2, 2), num_heads=[[16, 4], [16, 16]], win_size=[[27, 0], [27, 27]], groups=(8, 4))
+    torch.manual_seed(0)
+    plain = models.PCF_NATransformer(dtype=torch.bfloat16, **kw)
+    drop = models.PCF_NATransformer(dtype=torch.bfloat16, attn_drop=0.2, drop=0.1, **kw)
+    drop.load_state_dict(plain.state_dict())
+    plain, drop = plain.cuda(), drop.cuda()
+    x = torch.randn(4, 80, 200, generator=torch.Generator().manual_seed(1)).cuda()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        assert torch.equal(plain.eval()(x), drop.eval()(x))
+    x300 = torch.randn(4, 80, 300, generator=torch.Generator().manual_seed(2)).cuda()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        a, b = drop.train()(x300), drop(x300)
+    assert torch.isfinite(a).all() and not torch.equal(a, b)         # two draws of the masks
+    a.float().sum().backward()
+    g = drop.blocks[0].blocks[0].attn.qkv.weight.grad
+    assert g is not None and torch.isfinite(g).all() and g.abs().sum() > 0
