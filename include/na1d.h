@@ -165,6 +165,28 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb,
                                 void *workspace, int64_t workspace_bytes, void *stream);
 
 /*
+ * The fused operator with attention dropout: replaces nn.Dropout(attn_drop) between the softmax and the second
+ * contraction (models/PCF_NATransformer.py:71,149; every configuration of the reference sets attn_drop = 0, which is
+ * what na1d_fused_forward / na1d_fused_backward compute).  Probability (b, t, j) - packed sequence b, query row t,
+ * window slot j - is kept iff
+ *     mix32(key ^ (j * 0x9E3779B9)) >= floor(p_drop * 2^32),
+ *     key = mix32(mix32(lo32(row) ^ lo32(seed)) + hi32(row) * 0x9E3779B9 + hi32(seed)),   row = b * T + t,
+ *     mix32(x): x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16   (32-bit arithmetic)
+ * and kept probabilities are scaled by 1 / (1 - p_drop); lse is that of the un-dropped softmax.  The mask is a pure
+ * function of (seed, b, t, j): the backward recomputes it from the same p_drop and seed, nothing is stored, and the
+ * stream differs from torch's (whose mask depends on its launch geometry).  0 <= p_drop < 1.  head_dim > 128
+ * returns NA1D_ERR_UNSUPPORTED for p_drop > 0.  All other arguments as in na1d_fused_forward / na1d_fused_backward.
+ */
+int na1d_fused_forward_dropout(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+                               const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
+                               int64_t left, float scale, int dtype, float p_drop, uint64_t seed, void *stream);
+int na1d_fused_backward_dropout(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+                                const void *out, const void *dout, const float *lse, const float *rpb,
+                                const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
+                                int64_t left, float scale, int dtype, float p_drop, uint64_t seed, void *workspace,
+                                int64_t workspace_bytes, void *stream);
+
+/*
  * Dense ("global") attention over whole sequences, forward and backward: replaces the body of the reference's
  * GlobalAttention.forward between the head split and the head merge (models/PCF_NATransformer.py:199-221),
  *     attn = softmax((q * scale) @ k^T + mask);  out = attn @ v

@@ -25,7 +25,9 @@ loops on tiny shapes, W=1 row dots, the dense ``q @ k^T`` embedding for
 the exact adjoint identities between P1/P2/P3, closed-form masks, library
 softmax on the valid slots, and ``torch.autograd.gradcheck`` in fp64; the dense
 attention by index loops, ``F.scaled_dot_product_attention`` with the same mask,
-the closed-form mask, the full-window NA1D it must agree with, and gradcheck.
+the closed-form mask, the full-window NA1D it must agree with, and gradcheck; the
+dropout hash by a C program compiled from an independent transcription of the rule
+in include/na1d.h, bijectivity of the finaliser, and keep-rate / independence statistics.
 No function here is "parity unpinned".
 
 Layout everywhere: ``q, k, v : [B, T, C]`` with ``B = N * H`` (batch major,
@@ -34,6 +36,7 @@ addresses key ``t - left + j`` (``t + (j - left) * dilation`` when dilated).
 """
 from __future__ import annotations
 
+import numpy as np
 import torch
 import torch.nn.functional as F
 
@@ -135,15 +138,48 @@ def logits(q, k, W, left, rpb=None, padding=None, num_heads=1, dilation=1):
     return z.view(B, T, W)
 
 
-def na1d_forward(q, k, v, W, left, rpb=None, padding=None, num_heads=1, dilation=1):
-    """Full NA1D: returns ``(O, P, LSE)``; ``q`` is expected pre-scaled (:141)."""
+def _mix32(x):
+    """The 32-bit finaliser of the dropout hash on a uint32 array (wrapping arithmetic)."""
+    x = x ^ (x >> np.uint32(16))
+    x = x * np.uint32(0x7FEB352D)
+    x = x ^ (x >> np.uint32(15))
+    x = x * np.uint32(0x846CA68B)
+    return x ^ (x >> np.uint32(16))
+
+
+def dropout_keep(B, T, W, p, seed):
+    """bool ``[B, T, W]``: which probabilities the fused operator's attention dropout keeps - the rule stated
+    in include/na1d.h for na1d_fused_forward_dropout, a hash of (seed, row = b*T + t, slot j) against
+    ``floor(p * 2^32)``.  Stands where the reference has nn.Dropout (models/PCF_NATransformer.py:71,149);
+    the random stream is this library's own, the distribution (independent, keep rate 1 - p) is the reference's.
+    """
+    return torch.from_numpy(dropout_keep_rows(np.arange(B * T, dtype=np.uint64), W, p, seed)).view(B, T, W)
+
+
+def dropout_keep_rows(row, W, p, seed):
+    """The same for explicit row numbers ``b*T + t`` (uint64 array) -> bool ``[len(row), W]``."""
+    gold = np.uint32(0x9E3779B9)
+    with np.errstate(over="ignore"):
+        row = np.asarray(row, dtype=np.uint64)
+        lo, hi = (row & np.uint64(0xFFFFFFFF)).astype(np.uint32), (row >> np.uint64(32)).astype(np.uint32)
+        key = _mix32(_mix32(lo ^ np.uint32(seed & 0xFFFFFFFF)) + hi * gold + np.uint32((seed >> 32) & 0xFFFFFFFF))
+        h = _mix32(key[:, None] ^ (np.arange(W, dtype=np.uint32) * gold)[None, :])
+    threshold = min(int(p * 4294967296.0), 0xFFFFFFFF)
+    return h >= np.uint32(threshold)
+
+
+def na1d_forward(q, k, v, W, left, rpb=None, padding=None, num_heads=1, dilation=1, keep=None, p_drop=0.0):
+    """Full NA1D: returns ``(O, P, LSE)``; ``q`` is expected pre-scaled (:141).  With ``keep`` (bool
+    ``[B,T,W]``) the probabilities go through dropout before the second contraction (:149): ``O = (keep * P /
+    (1 - p_drop)) . V``; the returned ``P`` and ``LSE`` are those of the softmax."""
     z = logits(q, k, W, left, rpb, padding, num_heads, dilation)
     p = torch.softmax(z, dim=-1)
     lse = torch.logsumexp(z, dim=-1)
-    return av_band(p, v, W, left, dilation), p, lse
+    pd = p if keep is None else p * keep.to(p.dtype) / (1.0 - p_drop)
+    return av_band(pd, v, W, left, dilation), p, lse
 
 
-def na1d_backward(q, k, v, do, W, left, rpb=None, padding=None, num_heads=1, dilation=1):
+def na1d_backward(q, k, v, do, W, left, rpb=None, padding=None, num_heads=1, dilation=1, keep=None, p_drop=0.0):
     """Gradients by ``torch.autograd`` through :func:`na1d_forward`.
 
     Returns ``(dq, dk, dv, drpb)`` with ``drpb`` shaped ``[H, W]`` (``None`` without bias).
@@ -155,7 +191,7 @@ def na1d_backward(q, k, v, do, W, left, rpb=None, padding=None, num_heads=1, dil
     if rpb is not None:
         rpb = rpb.detach().clone().requires_grad_(True)
         leaves.append(rpb)
-    o, _, _ = na1d_forward(q, k, v, W, left, rpb, padding, num_heads, dilation)
+    o, _, _ = na1d_forward(q, k, v, W, left, rpb, padding, num_heads, dilation, keep, p_drop)
     grads = torch.autograd.grad(o, leaves, do)
     drpb = grads[3].reshape(num_heads, W) if rpb is not None else None
     return grads[0], grads[1], grads[2], drpb

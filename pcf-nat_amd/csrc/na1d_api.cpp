@@ -229,6 +229,44 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb, const
                           (float *)workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
 }
 
+int na1d_fused_forward_dropout(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+                               const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
+                               int64_t left, float scale, int dtype, float p_drop, uint64_t seed, void *stream) {
+    NA1D_CHECK(out, q, k, B, T, C, W, left, H, dtype, g);
+    if (!v) return NA1D_ERR_NULL;
+    if (misaligned(v)) return NA1D_ERR_ALIGN;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
+    g.drop = na1d::make_dropout(p_drop, seed);
+    const na1d::Layout packed = na1d::packed_layout(g);
+    const int st = mfma_allowed() ? mfma_fused_fwd(out, lse, q, k, v, rpb, t_valid, g, packed, packed, scale, dtype,
+                                                   (hipStream_t)stream)
+                                  : NA1D_ERR_UNSUPPORTED;
+    if (st != NA1D_ERR_UNSUPPORTED) return st;
+    return na1d::generic::fused_fwd(out, lse, q, k, v, rpb, t_valid, g, scale, dtype, (hipStream_t)stream);
+}
+
+int na1d_fused_backward_dropout(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+                                const void *out, const void *dout, const float *lse, const float *rpb,
+                                const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
+                                int64_t left, float scale, int dtype, float p_drop, uint64_t seed, void *workspace,
+                                int64_t workspace_bytes, void *stream) {
+    NA1D_CHECK(dq, q, k, B, T, C, W, left, H, dtype, g);
+    if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
+    if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
+        return NA1D_ERR_ALIGN;
+    if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
+    g.drop = na1d::make_dropout(p_drop, seed);
+    const na1d::Layout packed = na1d::packed_layout(g);
+    const int st = mfma_allowed() ? mfma_fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g,
+                                                   packed, packed, scale, dtype, (float *)workspace,
+                                                   workspace ? workspace_bytes : 0, (hipStream_t)stream)
+                                  : NA1D_ERR_UNSUPPORTED;
+    if (st != NA1D_ERR_UNSUPPORTED) return st;
+    return na1d::generic::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, scale, dtype,
+                                    (hipStream_t)stream);
+}
+
 int na1d_global_forward(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
                         int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, void *stream) {
     NA1D_CHECK(out, q, k, B, T, C, 1, 0, H, dtype, g);

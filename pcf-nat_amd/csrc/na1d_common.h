@@ -65,11 +65,49 @@ __device__ inline Chunk8 pack8(const float (&f)[8]) {
 
 __device__ inline float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
 
+// Attention dropout of the fused operator.  Whether probability (b, t, j) - packed sequence b, query row t,
+// window slot j - survives is a pure function of (seed, b * T + t, j), so that the forward, the backward and any
+// kernel variant agree without storing a mask:
+//     key  = mix32(mix32(lo32(row) ^ lo32(seed)) + hi32(row) * 0x9E3779B9 + hi32(seed)),   row = b * T + t
+//     keep = mix32(key ^ (j * 0x9E3779B9)) >= threshold,                                   threshold = floor(p * 2^32)
+// with mix32 the 32-bit finaliser x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16.
+// Survivors are scaled by 1 / (1 - p).  threshold 0 switches it off.
+struct Dropout {
+    uint32_t threshold = 0, seed_lo = 0, seed_hi = 0;
+    float inv_keep = 1.f;
+};
+inline Dropout make_dropout(float p, uint64_t seed) {
+    Dropout d;
+    if (p > 0.f) {
+        const double t = (double)p * 4294967296.0;
+        d.threshold = t >= 4294967295.0 ? 0xffffffffu : (uint32_t)t;
+        d.seed_lo = (uint32_t)seed;
+        d.seed_hi = (uint32_t)(seed >> 32);
+        d.inv_keep = (float)(1.0 / (1.0 - (double)p));
+    }
+    return d;
+}
+__host__ __device__ inline uint32_t mix32(uint32_t x) {
+    x ^= x >> 16;
+    x *= 0x7feb352du;
+    x ^= x >> 15;
+    x *= 0x846ca68bu;
+    x ^= x >> 16;
+    return x;
+}
+__host__ __device__ inline uint32_t dropout_row_key(uint64_t row, const Dropout &d) {
+    return mix32(mix32((uint32_t)row ^ d.seed_lo) + (uint32_t)(row >> 32) * 0x9E3779B9u + d.seed_hi);
+}
+__host__ __device__ inline bool dropout_keeps(uint32_t row_key, int slot, const Dropout &d) {
+    return mix32(row_key ^ ((uint32_t)slot * 0x9E3779B9u)) >= d.threshold;
+}
+
 // Problem description shared by every launcher.
 struct Geom {
     int64_t B, T;
     int C, W, L;      // head_dim, window, left
     int H;            // heads (B % H == 0); 1 for the un-fused entry points
+    Dropout drop;     // fused operator only; off by default
 };
 
 // Element strides of a [samples, heads, T, C] view of a tensor whose channels are contiguous.  The packed

@@ -310,6 +310,7 @@ int gather(void *out, const float *attn, const void *x, const Geom &g, int dtype
 
 int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
               const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s) {
+    if (g.drop.threshold) return NA1D_ERR_UNSUPPORTED;      // dropout lives in the matrix-core kernels only
     const int64_t rows = g.B * g.T;
     const int64_t blocks = (rows + kFwdRows - 1) / kFwdRows;
     if (blocks > 0x7fffffffLL) return NA1D_ERR_SHAPE;
@@ -323,6 +324,7 @@ int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v
 int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
               const void *out, const void *dout, const float *lse, const float *rpb,
               const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s) {
+    if (g.drop.threshold) return NA1D_ERR_UNSUPPORTED;
     int R = 32;
     auto bytes = [&](int r) { return (size_t)(2 * (r + g.W - 1) * g.W + (r + g.W - 1)) * sizeof(float); };
     while (R > 8 && bytes(R) > 60 * 1024) R /= 2;

@@ -8,18 +8,19 @@ namespace mfma {
 // =============================================================================
 // Fused forward
 // =============================================================================
-template <class DT, int C, int NBV>
+template <class DT, int C, int NBV, bool DROP>
 __global__ void __launch_bounds__(kThreads)
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale, uint32_t strips_magic, uint32_t heads_magic, Strides in, Strides outl,
-                 int shift) {
+                 int shift, Dropout drop) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = Strip<C>::kMaxTiles;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
     // dynamic LDS (launch_fwd): K and V regions of nt+2 tiles starting one tile before the strip (row 16*i0 - 16:
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
     // forward is not short of LDS), Q region of nt tiles
@@ -126,10 +127,20 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
             py[r] = __builtin_amdgcn_exp2f(zy[r] - m);
             sum += px[r] + py[r];
         }
+        if constexpr (DROP) {                    // dropped probabilities leave the sum as it is and O without them
+            const uint32_t key = dropout_row_key((uint64_t)b * T + qrow, drop);
+            const int j0 = 4 * g - n + L - shift;                    // window slot of register 0 of set X
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int jx = j0 + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0);
+                px[r] = dropout_keeps(key, jx, drop) ? px[r] : 0.f;
+                py[r] = dropout_keeps(key, j0 + r + 16, drop) ? py[r] : 0.f;
+            }
+        }
         const u32x2 pkx = {Mma<DT>::pack(px[0], px[1]), Mma<DT>::pack(px[2], px[3])};
         const u32x2 pky = {Mma<DT>::pack(py[0], py[1]), Mma<DT>::pack(py[2], py[3])};
         sum = xor_sum(sum);
-        const float inv = __builtin_amdgcn_rcpf(sum);
+        const float inv = __builtin_amdgcn_rcpf(sum) * (DROP ? drop.inv_keep : 1.f);
 
         // O^T = sum over blocks of V_blk^T . P^T
         u32x2 pb[NBV];
@@ -166,12 +177,15 @@ int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *
                const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &outl, float scale, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
-    auto kern = window_blocks(g) == 2 ? fused_fwd_kernel<DT, C, 2> : fused_fwd_kernel<DT, C, 3>;
+    const bool two = window_blocks(g) == 2;
+    auto kern = g.drop.threshold ? (two ? fused_fwd_kernel<DT, C, 2, true> : fused_fwd_kernel<DT, C, 3, true>)
+                                 : (two ? fused_fwd_kernel<DT, C, 2, false> : fused_fwd_kernel<DT, C, 3, false>);
     const size_t lds = (size_t)2 * region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
-                  div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g));
+                  div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g),
+                  g.drop);
     return launch_status();
 }
 
@@ -228,20 +242,21 @@ template <int C> struct StripBwd {
 #endif
 };
 
-template <class DT, int C, int NBV>
+template <class DT, int C, int NBV, bool DROP>
 __global__ void __launch_bounds__(kThreads)
 fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, float *__restrict__ drpb,
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes, uint32_t strips_magic,
-                 uint32_t heads_magic, Strides in, Strides outl, int shift) {
+                 uint32_t heads_magic, Strides in, Strides outl, int shift, Dropout drop) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
                    drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width,
                    outl.sample, outl.head, outl.pitch, outl.width, shift);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
     constexpr int kRowsQ = (MT + 2) * 16;
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
@@ -361,6 +376,23 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         for (int r = 0; r < 4; ++r) {
             px[r] = __builtin_amdgcn_exp2f(zx[r]);
             py[r] = __builtin_amdgcn_exp2f(zy[r]);
+        }
+        // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dV takes D*P and dP = D * (dO . V^T).
+        float fx[4] = {1.f, 1.f, 1.f, 1.f}, fy[4] = {1.f, 1.f, 1.f, 1.f};
+        if constexpr (DROP) {
+            const uint32_t key = dropout_row_key((uint64_t)b * T + qrow, drop);
+            const int j0 = 4 * g - n + L - shift;                    // window slot of register 0 of set X
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int jx = j0 + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0);
+                fx[r] = dropout_keeps(key, jx, drop) ? drop.inv_keep : 0.f;
+                fy[r] = dropout_keeps(key, j0 + r + 16, drop) ? drop.inv_keep : 0.f;
+                dpx[r] *= fx[r];
+                dpy[r] *= fy[r];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
             part = __builtin_fmaf(px[r], dpx[r], part);
             part = __builtin_fmaf(py[r], dpy[r], part);
         }
@@ -370,6 +402,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         for (int r = 0; r < 4; ++r) {
             dsx[r] = px[r] * (dpx[r] - delta);
             dsy[r] = py[r] * (dpy[r] - delta);
+            if constexpr (DROP) {      // the probability as the forward used it
+                px[r] *= fx[r];
+                py[r] *= fy[r];
+            }
         }
         sc[jt][0][0] = u32x2{Mma<DT>::pack(px[0], px[1]), Mma<DT>::pack(px[2], px[3])};
         sc[jt][1][0] = u32x2{Mma<DT>::pack(py[0], py[1]), Mma<DT>::pack(py[2], py[3])};
@@ -519,7 +555,9 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
     float *partial = nullptr;
     if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
-    auto kern = window_blocks(g) == 2 ? fused_bwd_kernel<DT, C, 2> : fused_bwd_kernel<DT, C, 3>;
+    const bool two = window_blocks(g) == 2;
+    auto kern = g.drop.threshold ? (two ? fused_bwd_kernel<DT, C, 2, true> : fused_bwd_kernel<DT, C, 3, true>)
+                                 : (two ? fused_bwd_kernel<DT, C, 2, false> : fused_bwd_kernel<DT, C, 3, false>);
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
     const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + 2) * 4 * 512);
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
@@ -528,7 +566,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
-                  div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g));
+                  div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g), g.drop);
     if (partial && drpb)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();

@@ -40,18 +40,19 @@ __device__ inline float bias_at(LDS_PTR(float) bias_lds, int j, int W) {
 // =============================================================================
 // Forward
 // =============================================================================
-template <class DT, int C, int NBV>
+template <class DT, int C, int NBV, bool DROP>
 __global__ void __launch_bounds__(kThreads)
 wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                 const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                 const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                 int strips, float scale, uint32_t strips_magic, uint32_t heads_magic, Strides in, Strides outl,
-                int shift) {
+                int shift, Dropout drop) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = Strip<C>::kMaxTiles;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
     // dynamic LDS (launch_wide_fwd): K and V regions of kt tiles starting sb tiles before the strip, Q region of nt
     // tiles, kBiasSlots bias floats
     const int sb = (shift + 15) >> 4;                        // whole tiles in front of the strip
@@ -133,6 +134,7 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
         m = xor_max(m);
         float sum = 0.f;
         u32x2 pb[NBV];
+        const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, drop) : 0u;
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
             float p[4];
@@ -140,11 +142,13 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
             for (int r = 0; r < 4; ++r) {
                 p[r] = __builtin_amdgcn_exp2f(z[vb][r] - m);
                 sum += p[r];
+                // a dropped probability stays in the sum and leaves O
+                if (DROP && !dropout_keeps(drop_key, 16 * vb + 4 * g + r - shift - n + L, drop)) p[r] = 0.f;
             }
             pb[vb] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
         }
         sum = xor_sum(sum);
-        const float inv = __builtin_amdgcn_rcpf(sum);
+        const float inv = __builtin_amdgcn_rcpf(sum) * (DROP ? drop.inv_keep : 1.f);
 
         f32x4 o[CT];
 #pragma unroll
@@ -171,13 +175,13 @@ int launch_wide_fwd_n(void *out, float *lse, const void *q, const void *k, const
                       int shift, hipStream_t s) {
     const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
-    auto kern = wide_fwd_kernel<DT, C, NBV>;
+    auto kern = g.drop.threshold ? wide_fwd_kernel<DT, C, NBV, true> : wide_fwd_kernel<DT, C, NBV, false>;
     const int kt = sp.nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     const size_t lds = (size_t)2 * region_bytes<C>(kt) + region_bytes<C>(sp.nt) + kBiasSlots * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
-                  div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), shift);
+                  div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), shift, g.drop);
     return launch_status();
 }
 
@@ -226,20 +230,21 @@ inline WideBwdShape wide_bwd_shape(const WideCover &c) {
     return w;
 }
 
-template <class DT, int C, int NBV>
+template <class DT, int C, int NBV, bool DROP>
 __global__ void __launch_bounds__(kThreads)
 wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, float *__restrict__ drpb,
                 const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                 const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                 const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                 int strips, float scale, int kv_bytes, uint32_t strips_magic, uint32_t heads_magic, Strides in,
-                Strides outl, int shift) {
+                Strides outl, int shift, Dropout drop) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
                    kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width, outl.sample,
                    outl.head, outl.pitch, outl.width, shift);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
     const int hb = NBV - 1 - (shift >> 4), ha = (shift + 15) >> 4;
     const int qtiles = nt + hb + ha;                        // query-side tiles, <= kWideQueryTiles
     const int ktiles = qtiles + NBV - 1;                    // key-side tiles: whole virtual blocks
@@ -325,6 +330,8 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
         const int qrow = 16 * qt + n;
         const bool edge = s0 < 0 || s0 + 16 * NBV > tv;
         float p[NBV][4], dp[NBV][4], part = 0.f;
+        // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dV takes D*P and dP = D * (dO . V^T).
+        const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, drop) : 0u;
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
             RowOperand<C> kop, vop;
@@ -342,7 +349,9 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
                 }
                 p[vb][r] = __builtin_amdgcn_exp2f(z);
                 dp[vb][r] = d[r];
-                part = __builtin_fmaf(p[vb][r], d[r], part);
+                if constexpr (DROP)
+                    dp[vb][r] *= dropout_keeps(drop_key, 16 * vb + 4 * g + r - shift - n + L, drop) ? drop.inv_keep : 0.f;
+                part = __builtin_fmaf(p[vb][r], dp[vb][r], part);
             }
         }
         const float delta = xor_sum(part);
@@ -354,6 +363,8 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
             for (int r = 0; r < 4; ++r) {
                 ds[r] = p[vb][r] * (dp[vb][r] - delta);
                 if (own) racc[vb][r] += ds[r];
+                if constexpr (DROP)        // the probability as the forward used it
+                    p[vb][r] *= dropout_keeps(drop_key, 16 * vb + 4 * g + r - shift - n + L, drop) ? drop.inv_keep : 0.f;
             }
             sc[jt][vb][0] = u32x2{Mma<DT>::pack(p[vb][0], p[vb][1]), Mma<DT>::pack(p[vb][2], p[vb][3])};
             sc[jt][vb][1] = u32x2{Mma<DT>::pack(ds[0], ds[1]), Mma<DT>::pack(ds[2], ds[3])};
@@ -478,13 +489,13 @@ int launch_wide_bwd_n(void *dq, void *dk, void *dv, float *drpb, const void *q, 
     if (mt < 1) return NA1D_ERR_UNSUPPORTED;
     const Split sp = make_split(g.B, g.T, mt);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
-    auto kern = wide_bwd_kernel<DT, C, NBV>;
+    auto kern = g.drop.threshold ? wide_bwd_kernel<DT, C, NBV, true> : wide_bwd_kernel<DT, C, NBV, false>;
     const size_t lds = wide_bwd_lds<C>(sp.nt, NBV, w, kv_bytes);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, kv_bytes, div_magic(sp.strips), div_magic(g.H),
-                  byte_strides(in, g), byte_strides(outl, g), c.shift);
+                  byte_strides(in, g), byte_strides(outl, g), c.shift, g.drop);
     return launch_status();
 }
 

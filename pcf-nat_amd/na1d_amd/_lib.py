@@ -16,13 +16,14 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libna1d.so")
 
 BF16, FP16 = 0, 1
 
-_i64, _int, _f32, _ptr = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p
+_i64, _int, _f32, _ptr, _u64 = ctypes.c_int64, ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_uint64
 
 _UNFUSED = ("na1d_qk_forward", "na1d_av_forward", "na1d_q_backward", "na1d_k_backward",
             "na1d_a_backward", "na1d_v_backward")
 SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_backward_workspace_bytes",
                       "na1d_fused_forward_strided", "na1d_fused_backward_strided", "na1d_profile_events",
                       "na1d_global_forward", "na1d_global_backward", "na1d_global_backward_workspace_bytes",
+                      "na1d_fused_forward_dropout", "na1d_fused_backward_dropout",
                       "na1d_version", "na1d_status_string")
 UNSUPPORTED = -8
 
@@ -61,6 +62,10 @@ def load():
     lib.na1d_fused_backward_strided.argtypes = [_ptr] * 11 + [_i64] * 6 + [_f32, _int, _ptr, _ptr, _ptr, _i64, _ptr]
     lib.na1d_fused_backward_workspace_bytes.restype = _i64
     lib.na1d_fused_backward_workspace_bytes.argtypes = [_i64] * 6 + [_int]
+    lib.na1d_fused_forward_dropout.restype = _int
+    lib.na1d_fused_forward_dropout.argtypes = [_ptr] * 7 + [_i64] * 6 + [_f32, _int, _f32, _u64, _ptr]
+    lib.na1d_fused_backward_dropout.restype = _int
+    lib.na1d_fused_backward_dropout.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _f32, _u64, _ptr, _i64, _ptr]
     lib.na1d_global_forward.restype = _int
     lib.na1d_global_forward.argtypes = [_ptr] * 6 + [_i64] * 4 + [_f32, _int, _ptr]
     lib.na1d_global_backward.restype = _int
@@ -108,11 +113,17 @@ def call_unfused(name: str, out, a, b, B, T, C, W, left, dtype):
     check(st, name)
 
 
-def call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, H, T, C, W, left, scale):
+def call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, H, T, C, W, left, scale, dropout=None):
+    """``dropout``: ``None`` or ``(p, seed)`` for the entry point with attention dropout."""
     lib = load()
     with torch.cuda.device(out.device):
-        st = lib.na1d_fused_forward(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid),
-                                    B, H, T, C, W, left, scale, dtype_tag(q.dtype), _stream(out))
+        if dropout is None:
+            st = lib.na1d_fused_forward(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid),
+                                        B, H, T, C, W, left, scale, dtype_tag(q.dtype), _stream(out))
+        else:
+            st = lib.na1d_fused_forward_dropout(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid), B, H, T,
+                                                C, W, left, scale, dtype_tag(q.dtype), dropout[0], dropout[1],
+                                                _stream(out))
     check(st, "na1d_fused_forward")
 
 
@@ -124,14 +135,20 @@ def fused_backward_workspace_bytes(B, H, T, C, W, left, dtype) -> int:
 
 
 def call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, B, H, T, C, W, left, scale,
-                        workspace=None):
-    """``workspace``: optional uint8/any CUDA tensor used for the d rpb reduction."""
+                        workspace=None, dropout=None):
+    """``workspace``: optional uint8/any CUDA tensor used for the d rpb reduction; ``dropout`` as in the forward."""
     lib = load()
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with torch.cuda.device(dq.device):
-        st = lib.na1d_fused_backward(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(out), _p(dout),
-                                     _p(lse), _p(rpb), _p(t_valid), B, H, T, C, W, left, scale,
-                                     dtype_tag(q.dtype), _p(workspace), ws_bytes, _stream(dq))
+        if dropout is None:
+            st = lib.na1d_fused_backward(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(out), _p(dout),
+                                         _p(lse), _p(rpb), _p(t_valid), B, H, T, C, W, left, scale,
+                                         dtype_tag(q.dtype), _p(workspace), ws_bytes, _stream(dq))
+        else:
+            st = lib.na1d_fused_backward_dropout(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(out),
+                                                 _p(dout), _p(lse), _p(rpb), _p(t_valid), B, H, T, C, W, left, scale,
+                                                 dtype_tag(q.dtype), dropout[0], dropout[1], _p(workspace), ws_bytes,
+                                                 _stream(dq))
     check(st, "na1d_fused_backward")
 
 

@@ -52,8 +52,10 @@ def _strided_or_packed_backward(dq4, dk4, dv4, drpb, q4, k4, v4, packed_out, dou
 
 class _FusedNA1D(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, rpb, t_valid, num_heads, win_size, left, scale, deterministic, dilation):
+    def forward(ctx, q, k, v, rpb, t_valid, num_heads, win_size, left, scale, deterministic, dilation, dropout):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+        assert dropout is None or dilation == 1, "attention dropout is defined for dilation 1"
+        ctx.dropout = dropout
         assert q.dtype == k.dtype == v.dtype
         assert q.dim() == 3 and q.shape == k.shape == v.shape, "q, k, v must all be [B, T, C]"
         B, T, C = q.shape
@@ -68,7 +70,8 @@ class _FusedNA1D(torch.autograd.Function):
         ctx.geom = (num_heads, win_size, left, scale, deterministic, dilation)
         if dilation == 1:
             lse = torch.empty((B, T), dtype=torch.float32, device=q.device)
-            _lib.call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, num_heads, T, C, win_size, left, scale)
+            _lib.call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, num_heads, T, C, win_size, left, scale,
+                                    dropout=dropout)
             ctx.save_for_backward(q, k, v, out, rpb, t_valid, lse)
             return out
         # Dilation d: slot j of row t is row t + (j - left) * d, so the rows of one residue class t mod d only
@@ -102,7 +105,7 @@ class _FusedNA1D(torch.autograd.Function):
                     ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
         if dilation == 1:
             _lib.call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lses[0], rpb, t_valid,
-                                     B, num_heads, T, C, win_size, left, scale, workspace=ws)
+                                     B, num_heads, T, C, win_size, left, scale, workspace=ws, dropout=ctx.dropout)
         else:
             shape4 = (B // num_heads, num_heads, T, C)
             views = [z.view(shape4) for z in (dq, dk, dv, q, k, v, dout)]
@@ -112,11 +115,11 @@ class _FusedNA1D(torch.autograd.Function):
                                             _residue_lengths(t_valid, r, dilation), win_size, left, scale, ws)
         if drpb is not None:
             drpb = drpb.view(ctx.rpb_shape)
-        return dq, dk, dv, drpb, None, None, None, None, None, None, None
+        return dq, dk, dv, drpb, None, None, None, None, None, None, None, None
 
 
 def na1d_fused(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, scale=1.0, deterministic=False,
-               dilation=1):
+               dilation=1, dropout_p=0.0, seed=None):
     """Fused neighbourhood attention.
 
     q, k, v : contiguous ``[B, T, C]`` bf16/fp16, ``B = N * num_heads``.  ``q`` is
@@ -130,10 +133,20 @@ def na1d_fused(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, sca
               dq, dk, dv never use atomics.
     dilation : window slot j of row t addresses row ``t + (j - left) * dilation`` (the reference computes this on
               the CPU only, models/PCF_NATransformer.py:101-116,158-170; its CUDA path asserts dilation == 1).
+    dropout_p, seed : attention dropout inside the kernels (nn.Dropout(attn_drop) of models/PCF_NATransformer.py:71,149):
+              each probability is kept with chance ``1 - dropout_p`` and scaled by ``1 / (1 - dropout_p)``.  The mask
+              is a hash of (seed, sequence, row, window slot) that the backward recomputes; ``seed`` (a 64-bit int)
+              defaults to a draw from torch's CPU generator.  Needs ``dilation == 1`` and head_dim <= 128.
     Returns ``[B, T, C]`` in q's dtype.  The gradient of ``rpb`` has rpb's shape.
     """
+    dropout = None
+    if dropout_p > 0.0:
+        assert dropout_p < 1.0
+        if seed is None:
+            seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+        dropout = (float(dropout_p), int(seed))
     return _FusedNA1D.apply(q, k, v, rpb, t_valid, num_heads, win_size, left, float(scale), bool(deterministic),
-                            int(dilation))
+                            int(dilation), dropout)
 
 
 def na1d_fused_forward_lse(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, scale=1.0):

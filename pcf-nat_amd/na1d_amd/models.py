@@ -284,10 +284,8 @@ class NAttention(nn.Module):
         nn.init.normal_(self.relative_position_bias, mean=0.0, std=0.02)
         self.proj = _Projection.make(dim, dim, True, groups, channels_first)
         self.register_buffer("attn_mask", _window_mask(frames, win_size, left, None, torch.float32, "cpu").unsqueeze(1))
-        # The fused kernels never hold the probabilities in memory, so attention dropout (PCF :149; 0 in every
-        # configuration of the reference) is applied where the reference applies it: in the two-call chain.
-        self._chain = na == "unfused" or attn_drop > 0.0
-        if self._chain:         # like the reference's CUDA path, the two-call chain has no dilated kernels
+        assert attn_drop == 0.0 or dilation == 1, "attention dropout is built for dilation 1"
+        if na == "unfused":     # like the reference's CUDA path, the two-call chain has no dilated kernels
             self.NA1d_QK_Function, self.NA1d_AV_Function = getNA1dFunction(C=head_dim, dilation=dilation, dtype=dtype)
 
     def forward(self, x, padding=None):
@@ -303,7 +301,9 @@ class NAttention(nn.Module):
         extra = {} if self.dilation == 1 else {"dilation": self.dilation}
         if callable(self.na):
             out = self.na(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h, **extra)
-        elif self.na in ("fused", "fused_qkv") and not dropping:
+        elif self.na in ("fused", "fused_qkv"):              # dropout (PCF :149) happens inside the kernels
+            if dropping:
+                extra["dropout_p"] = self.attn_drop
             out = na1d_fused(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h, **extra)
         else:                                                # the reference's un-fused chain (:141-150)
             attn = self.NA1d_QK_Function.apply(q, k, w, left, 1).view(n, h, t, w)

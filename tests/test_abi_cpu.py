@@ -108,6 +108,21 @@ def test_strided_entry_points_validate():
     assert b(*bargs(ws=P(0x1008))) == -6
 
 
+def test_dropout_entry_points_validate():
+    lib = _lib.load()
+    ok = ctypes.c_void_p(0x1000)
+    f = lib.na1d_fused_forward_dropout
+    args = lambda **kw: [ok, None, ok, ok, kw.get("v", ok), None, None, kw.get("B", 4), 2, 8, kw.get("C", 16), 5, 2, 1.0, 0,
+                         kw.get("p", 0.5), 7, None]
+    assert f(*args(v=None)) == -1 and f(*args(C=20)) == -3 and f(*args(B=0)) == 0
+    assert f(*args(p=1.0)) == -5 and f(*args(p=-0.1)) == -5 and f(*args(p=float("nan"))) == -5
+    assert f(*args(C=136)) == -8                     # no dropout kernel above head_dim 128
+    b = lib.na1d_fused_backward_dropout
+    bargs = lambda **kw: [ok, ok, ok, None, ok, ok, ok, ok, ok, kw.get("lse", ok), None, None, 4, 2, 8, 16, 5, 2, 1.0, 0,
+                          kw.get("p", 0.5), 7, None, 0, None]
+    assert b(*bargs(lse=None)) == -1 and b(*bargs(p=1.5)) == -5
+
+
 def test_dense_attention_entry_points_validate():
     lib = _lib.load()
     P, ok = ctypes.c_void_p, ctypes.c_void_p(0x1000)

@@ -138,14 +138,15 @@ def test_mfa_nat_4x4_training_step_fp16(na):
     assert not torch.equal(before, gpu.fc.weight.detach())
 
 
-def test_attention_dropout_runs_through_the_two_call_chain():
+@pytest.mark.parametrize("na", ["fused", "fused_qkv", "unfused"])
+def test_attention_dropout_in_training_only(na):
     """attn_drop / drop of the reference's constructors (models/PCF_NATransformer.py:324,375; 0 in its
-    configurations): inactive in eval mode, and in training the probabilities are dropped where the reference
-    drops them, between the two calls of the un-fused chain."""
+    configurations): inactive in eval mode; in training the fused layers drop probabilities inside the kernels,
+    the un-fused chain between its two calls as the reference does (:149)."""
     kw = dict(depths=(2, 2), num_heads=[[16, 4], [16, 16]], win_size=[[27, 0], [27, 27]], groups=(8, 4))
     torch.manual_seed(0)
-    plain = models.PCF_NATransformer(dtype=torch.bfloat16, **kw)
-    drop = models.PCF_NATransformer(dtype=torch.bfloat16, attn_drop=0.2, drop=0.1, **kw)
+    plain = models.PCF_NATransformer(dtype=torch.bfloat16, na=na, **kw)
+    drop = models.PCF_NATransformer(dtype=torch.bfloat16, na=na, attn_drop=0.2, drop=0.1, **kw)
     drop.load_state_dict(plain.state_dict())
     plain, drop = plain.cuda(), drop.cuda()
     x = torch.randn(4, 80, 200, generator=torch.Generator().manual_seed(1)).cuda()

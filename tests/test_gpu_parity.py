@@ -553,3 +553,74 @@ def test_errors_become_python_exceptions():
         _lib.call_unfused("na1d_qk_forward", torch.empty(2, 8, 81, device="cuda"), q, q, 2, 8, 16, 81, 3, q.dtype)
     with pytest.raises(_lib.NA1DError):
         _lib.call_unfused("na1d_qk_forward", torch.empty(2, 8, 5, device="cuda"), q, q, 2, 8, 12, 5, 2, q.dtype)
+
+
+# --------------------------------------------------------------------------- attention dropout inside the kernels
+DROP_GEOMS = [  # (N, H, T, C, W, L): two-block, merged three-block, wide and lopsided windows, padded head dims, ragged tiles
+    (2, 2, 61, 32, 15, 7), (2, 4, 100, 16, 27, 13), (1, 2, 150, 64, 33, 16), (2, 1, 90, 32, 65, 32),
+    (2, 2, 47, 24, 9, 0), (1, 3, 130, 128, 17, 16), (2, 2, 5, 16, 27, 13), (1, 2, 300, 48, 80, 50),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", DROP_GEOMS, ids=lambda g: "x".join(map(str, g)))
+def test_fused_dropout_matches_oracle_with_the_same_mask(geom, dtype):
+    N, H, T, C, W, L = geom
+    B, p, seed = N * H, 0.3, 0x1234_5678_9ABC_DEF0
+    q, k, v, do = make_inputs(B, T, C, W, 51, dtype, n=4, scale=C ** -0.5)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(6)) * 0.5
+    pad = torch.tensor([0, T // 3][:N])
+    t_valid = (T - pad).to(torch.int32).cuda()
+    print("fused dropout", geom, dtype, flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    rd = rpb.cuda().requires_grad_(True)
+    out = na1d_fused(qd, kd, vd, W, L, rpb=rd, t_valid=t_valid, num_heads=H, dropout_p=p, seed=seed)
+    out.backward(do.cuda())
+
+    keep = O.dropout_keep(B, T, W, p, seed)
+    qf, kf, vf = q.float(), k.float(), v.float()
+    want_o, _, _ = O.na1d_forward(qf, kf, vf, W, L, rpb, pad, H, keep=keep, p_drop=p)
+    wq, wk, wv, wr = O.na1d_backward(qf, kf, vf, do.float(), W, L, rpb, pad, H, keep=keep, p_drop=p)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float(), want_o) < tol, "O"
+    assert O.rel_l2(qd.grad.float(), wq) < tol, "dQ"
+    assert O.rel_l2(kd.grad.float(), wk) < tol, "dK"
+    assert O.rel_l2(vd.grad.float(), wv) < tol, "dV"
+    assert _err(rd.grad, wr) < tol, "drpb"
+    # the dropped operator is not the plain one, and the same seed gives the same bits
+    plain = na1d_fused(qd.detach(), kd.detach(), vd.detach(), W, L, rpb=rpb.cuda(), t_valid=t_valid, num_heads=H)
+    again = na1d_fused(qd.detach(), kd.detach(), vd.detach(), W, L, rpb=rpb.cuda(), t_valid=t_valid, num_heads=H,
+                       dropout_p=p, seed=seed)
+    assert torch.equal(again, out) and not torch.equal(plain, out)
+
+
+@pytest.mark.parametrize("W,L", [(15, 7), (27, 13), (65, 32), (31, 3)])
+def test_dropout_mask_is_bit_exact(W, L):
+    """One-hot values turn the output into the dropped probability matrix itself: with zero queries every
+    in-range slot has a positive probability, so out[t, u] != 0 exactly where slot u - t + L of row t is kept."""
+    B, T, C, p, seed = 3, 100, 128, 0.5, 99
+    q = torch.zeros(B, T, C, dtype=torch.float16, device="cuda")
+    v = torch.zeros(B, T, C, dtype=torch.float16)
+    v[:, torch.arange(T), torch.arange(T)] = 1.0
+    out = na1d_fused(q, q, v.cuda(), W, L, dropout_p=p, seed=seed).cpu()
+    keep = O.dropout_keep(B, T, W, p, seed)
+    want = torch.zeros(B, T, C, dtype=torch.bool)
+    for j in range(W):
+        lo, hi = max(0, L - j), min(T, T + L - j)
+        rows = torch.arange(lo, hi)
+        want[:, rows, rows - L + j] = keep[:, lo:hi, j]
+    assert torch.equal(out != 0, want)
+    kept = out[out != 0].float()
+    assert ((kept * (1 - p) * W).round() >= 1).all()                 # survivors carry 1 / (1 - p)
+
+
+def test_dropout_rate_zero_is_the_plain_operator_and_bad_rates_are_rejected():
+    q, k, v = dev(*make_inputs(4, 50, 32, 15, 3, torch.bfloat16))
+    assert torch.equal(na1d_fused(q, k, v, 15, 7, dropout_p=0.0), na1d_fused(q, k, v, 15, 7))
+    out = torch.empty_like(q)
+    with pytest.raises(_lib.NA1DError):
+        _lib.call_fused_forward(out, None, q, k, v, None, None, 4, 1, 50, 32, 15, 7, 1.0, dropout=(1.0, 1))
+    wide = torch.zeros(2, 8, 136, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.NA1DError):                               # head_dim > 128 has no dropout kernels
+        _lib.call_fused_forward(torch.empty_like(wide), None, wide, wide, wide, None, None, 2, 1, 8, 136, 5, 2, 1.0,
+                                dropout=(0.5, 1))

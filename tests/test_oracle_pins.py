@@ -328,3 +328,101 @@ def test_global_gradcheck_fp64():
     assert torch.allclose(dv, torch.einsum("btu,btc->buc", p, do), atol=1e-12)
     assert torch.allclose(dq, 0.4 * torch.einsum("btu,buc->btc", ds, k.detach()), atol=1e-12)
     assert torch.allclose(dk, 0.4 * torch.einsum("btu,btc->buc", ds, q.detach()), atol=1e-12)
+
+
+# --------------------------------------------------------------------------
+# attention dropout of the fused operator
+# --------------------------------------------------------------------------
+_DROPOUT_C = r"""
+/* keep rule of na1d_fused_forward_dropout, transcribed from its statement in the public header */
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+static uint32_t mix(uint32_t x) { x ^= x >> 16; x *= 0x7feb352dU; x ^= x >> 15; x *= 0x846ca68bU; x ^= x >> 16; return x; }
+int main(int argc, char **argv) {
+    uint64_t seed = strtoull(argv[1], 0, 10);
+    uint32_t threshold = (uint32_t)strtoull(argv[2], 0, 10);
+    int W = atoi(argv[3]);
+    for (int a = 4; a < argc; ++a) {
+        uint64_t row = strtoull(argv[a], 0, 10);
+        uint32_t key = mix(mix((uint32_t)row ^ (uint32_t)seed) + (uint32_t)(row >> 32) * 0x9E3779B9U + (uint32_t)(seed >> 32));
+        for (int j = 0; j < W; ++j) putchar(mix(key ^ ((uint32_t)j * 0x9E3779B9U)) >= threshold ? '1' : '0');
+        putchar('\n');
+    }
+    return 0;
+}
+"""
+
+
+def test_dropout_hash_matches_a_c_transcription(tmp_path):
+    import subprocess
+    import numpy as np
+    src = tmp_path / "keep.c"
+    src.write_text(_DROPOUT_C)
+    exe = tmp_path / "keep"
+    subprocess.run(["gcc", "-O1", "-o", str(exe), str(src)], check=True)
+    rows = [0, 1, 2, 299, 300, 2 ** 31, 2 ** 32 - 1, 2 ** 32, 2 ** 32 + 1, 2 ** 40 + 5, 2 ** 63 + 12345]
+    for seed, p in ((0, 0.5), (12345678901234567, 0.1), (2 ** 64 - 1, 0.9), (77, 1e-9)):
+        thr = min(int(p * 4294967296.0), 0xFFFFFFFF)
+        out = subprocess.run([str(exe), str(seed), str(thr), "80"] + [str(r) for r in rows], check=True,
+                             capture_output=True, text=True).stdout.split()
+        want = np.array([[c == "1" for c in line] for line in out])
+        got = O.dropout_keep_rows(np.array(rows, dtype=np.uint64), 80, p, seed)
+        assert (got == want).all()
+    assert O.dropout_keep(3, 5, 7, 0.0, 9).all()                      # threshold 0 keeps everything
+    full = O.dropout_keep(3, 5, 7, 0.25, 9)
+    assert (full.view(15, 7).numpy() == O.dropout_keep_rows(np.arange(15), 7, 0.25, 9)).all()   # row = b*T + t
+
+
+def test_dropout_finaliser_is_a_bijection():
+    import numpy as np
+    def unshift(y, s):                       # inverse of x ^= x >> s
+        x = y.copy()
+        for _ in range(32 // s + 1):
+            x = y ^ (x >> np.uint32(s))
+        return x
+    rng = np.random.default_rng(0)
+    x = rng.integers(0, 2 ** 32, 1 << 16, dtype=np.uint32)
+    with np.errstate(over="ignore"):
+        y = O._mix32(x)
+        z = unshift(y, 16) * np.uint32(pow(0x846CA68B, -1, 2 ** 32))
+        z = unshift(z, 15) * np.uint32(pow(0x7FEB352D, -1, 2 ** 32))
+        z = unshift(z, 16)
+    assert (z == x).all()
+    assert O._mix32(np.zeros(1, dtype=np.uint32))[0] == 0            # the one fixed point the construction implies
+
+
+def test_dropout_mask_statistics():
+    B, T, W = 16, 300, 27
+    n = B * T * W
+    for p in (0.1, 0.5, 0.8):
+        keep = O.dropout_keep(B, T, W, p, 2024).double()
+        sigma = (p * (1 - p) / n) ** 0.5
+        assert abs(keep.mean().item() - (1 - p)) < 5 * sigma
+        c = keep - keep.mean()
+        var = (c * c).mean()
+        for a, b in ((c[:, :, 1:], c[:, :, :-1]), (c[:, 1:], c[:, :-1]), (c[1:], c[:-1])):   # slots, rows, sequences
+            assert abs(((a * b).mean() / var).item()) < 5 / n ** 0.5 * 2
+        other = O.dropout_keep(B, T, W, p, 2025).double()
+        assert abs(((other - other.mean()) * c).mean().item() / var.item()) < 10 / n ** 0.5      # seeds are unrelated
+
+
+def test_forward_with_dropout_matches_index_loops_and_differentiates():
+    B, T, C, W, L, p = 2, 7, 3, 5, 2, 0.4
+    q, k, v = _rand(B, T, C), _rand(B, T, C), _rand(B, T, C)
+    keep = O.dropout_keep(B, T, W, p, 3)
+    assert 0 < keep.sum() < keep.numel()
+    o, prob, _ = O.na1d_forward(q, k, v, W, L, keep=keep, p_drop=p)
+    o_plain, prob_plain, _ = O.na1d_forward(q, k, v, W, L)
+    assert torch.equal(prob, prob_plain)                              # the softmax is not renormalised
+    for b in range(B):
+        for t in range(T):
+            want = torch.zeros(C, dtype=F64)
+            for j in range(W):
+                u = t - L + j
+                if 0 <= u < T and keep[b, t, j]:
+                    want += prob[b, t, j] / (1 - p) * v[b, u]
+            assert torch.allclose(o[b, t], want, atol=1e-12)
+    q, k, v = (x.requires_grad_(True) for x in (q, k, v))
+    assert torch.autograd.gradcheck(lambda a, b_, c: O.na1d_forward(a, b_, c, W, L, keep=keep, p_drop=p)[0], (q, k, v),
+                                    atol=1e-7)
