@@ -128,6 +128,16 @@ class TDNNBlock(nn.Module):
     def forward(self, x):
         return self.norm(self.activation(self.conv(x)))
 
+    def forward_tokens(self, x, pre_norm=None):
+        """Inference on ``[N, T, C]`` (kernel size 1): one matrix product over all tokens, a batch norm in front
+        (`pre_norm`) folded into it, the one behind applied as its per-channel affine map."""
+        w, b, a, c = _prepared(
+            self, "tokens", x,
+            lambda: (_fold_norm(pre_norm, self.conv) if pre_norm is not None else (_dense_weight(self.conv), self.conv.bias))
+            + _bn_affine(self.norm),
+            deps=[self.conv.weight, self.conv.bias] + _bn_tensors(self.norm) + (_bn_tensors(pre_norm) if pre_norm else []))
+        return torch.addcmul(c, F.relu(F.linear(x, w, b)), a)
+
 
 def _length_mask(shape, lens):
     n, _, t = shape
@@ -163,6 +173,36 @@ class AttentiveStatisticsPooling(nn.Module):
         std = torch.sqrt((w * (x - mean).pow(2)).sum(-1, keepdim=True).clamp(self.eps))
         return torch.cat((mean, std), dim=1).squeeze(-1)
 
+    def forward_tokens(self, x, lens=None):
+        """The same pooling in inference on ``[N, T, C]``: reductions over T run down the columns, and the context
+        ``[x, mean, std]`` is never concatenated - the first convolution is split into its three column blocks and
+        the mean / std blocks, constant along T, are applied once per utterance."""
+        n, t, c = x.shape
+        if lens is None:
+            mask = None
+            mean = x.mean(1, keepdim=True)
+            std = torch.sqrt(x.var(1, keepdim=True).clamp(self.eps))
+        else:
+            count = torch.round(lens * t).view(n, 1, 1)
+            mask = torch.arange(t, device=x.device).view(1, t, 1) < count
+            mean = (x * mask).sum(1, keepdim=True) / count
+            std = torch.sqrt((((x - mean).pow(2) * mask).sum(1, keepdim=True) / count).clamp(self.eps))
+        tdnn = self.tdnn
+        w, b, a, d, w2, b2 = _prepared(
+            self, "tokens", x,
+            lambda: (_dense_weight(tdnn.conv), tdnn.conv.bias) + _bn_affine(tdnn.norm) + (_dense_weight(self.conv), self.conv.bias),
+            deps=[tdnn.conv.weight, tdnn.conv.bias, self.conv.weight, self.conv.bias] + _bn_tensors(tdnn.norm))
+        dt = w.dtype
+        const = F.linear(mean.to(dt), w[:, c:2 * c]) + F.linear(std.to(dt), w[:, 2 * c:], b)        # [N, 1, A]
+        h = torch.addcmul(d, F.relu(F.linear(x.to(dt), w[:, :c]) + const), a)
+        logits = F.linear(torch.tanh(h), w2, b2).float()
+        if mask is not None:
+            logits = logits.masked_fill(~mask, -torch.inf)
+        p = F.softmax(logits, dim=1)
+        mean = (p * x).sum(1, keepdim=True)
+        std = torch.sqrt((p * (x - mean).pow(2)).sum(1, keepdim=True).clamp(self.eps))
+        return torch.cat((mean, std), dim=2).squeeze(1)
+
 
 class StatisticsPooling(nn.Module):
     def __init__(self):
@@ -178,6 +218,9 @@ class StatisticsPooling(nn.Module):
             mean = (x * mask).sum(-1, keepdim=True) / count
             std = torch.sqrt((((x - mean).pow(2) * mask).sum(-1, keepdim=True) / count).clamp(self.eps))
         return torch.cat([mean, std], dim=1).squeeze(-1)
+
+    def forward_tokens(self, x, lens=None):
+        return self.forward(x.transpose(1, 2), lens)
 
 
 # --------------------------------------------------------------------------- attention
@@ -212,18 +255,41 @@ def _merge_heads(x, n, num_heads, channels_first):
     return x.transpose(1, 2).contiguous().view(n, t, num_heads * hd)
 
 
-def _prepared(module, tag, like, build):
+def _prepared(module, tag, like, build, deps=None):
     """`build()` -> tuple of tensors derived from `module`'s parameters (dense / reordered weights, biases), cast
     to the dtype the product on `like` runs in.  While autograd is recording they are rebuilt every call (the
-    gradient has to reach the parameters); otherwise they are kept until a parameter changes."""
+    gradient has to reach the parameters); otherwise they are kept until a parameter changes.  `deps`: the
+    tensors `build` reads, when they are not just the module's own parameters."""
     dt = _compute_dtype(like)
-    if torch.is_grad_enabled() and any(p.requires_grad for p in module.parameters(recurse=False)):
+    deps = list(module.parameters(recurse=False)) if deps is None else [d for d in deps if d is not None]
+    if torch.is_grad_enabled() and any(p.requires_grad for p in deps):
         return tuple(None if t is None else t.to(dt) for t in build())
-    key = (tag, dt) + tuple((p.data_ptr(), p._version) for p in module.parameters(recurse=False))
+    key = (tag, dt) + tuple((p.data_ptr(), p._version) for p in deps)
     cache = module.__dict__.setdefault("_prepared_cache", {})
     if cache.get("key") != key:
         cache["key"], cache["val"] = key, tuple(None if t is None else t.detach().to(dt) for t in build())
     return cache["val"]
+
+
+def _bn_affine(bn):
+    """Inference-mode batch norm as ``y = x * a + b`` per channel, in fp32."""
+    a = bn.weight.float() * torch.rsqrt(bn.running_var.float() + bn.eps)
+    return a, bn.bias.float() - bn.running_mean.float() * a
+
+
+def _bn_tensors(bn):
+    return [bn.weight, bn.bias, bn.running_mean, bn.running_var]
+
+
+def _fold_norm(bn, proj, order=None):
+    """Weight and bias (fp32) of ``proj(bn(x))`` as one affine map on tokens: ``W diag(a)`` and ``W b + bias``;
+    `order` permutes the output channels."""
+    a, b = _bn_affine(bn)
+    w = _dense_weight(proj).float()
+    bias = proj.bias.float() if proj.bias is not None else torch.zeros(w.shape[0], device=w.device)
+    if order is not None:
+        w, bias = w.index_select(0, order), bias.index_select(0, order)
+    return w * a, bias + w @ b
 
 
 def _compute_dtype(x):
@@ -415,6 +481,51 @@ class NATFLayer(nn.Module):
         x = x + self.drop_path(y)
         return x + self.drop_path(self.mlp(self.norm2(x)))
 
+    def tokens_ok(self):
+        """Whether :meth:`forward_tokens` serves this layer."""
+        return self.attn.na == "fused_qkv" if self.local else self.attn.dense == "native"
+
+    def forward_tokens(self, x, padding=None, pos_emb=None, masked=False):
+        """The layer in inference on token-major ``x [N, T, C]`` (``pos_emb [1, T, C]``), whatever the layout of
+        the model: the same parameters, with each batch norm folded into the projection that follows it (running
+        statistics make it a per-channel affine map), every projection one matrix product over all N*T tokens
+        with its bias in the epilogue, and the attention operators reading and writing the token-major tensors
+        in place.  ``masked``: the global layers mask the padded rows and columns."""
+        n, t, dim = x.shape
+        attn, h = self.attn, self.attn.num_heads
+        bn1 = self.norm1.norm if isinstance(self.norm1, TokenBatchNorm) else self.norm1
+        bn2 = self.norm2.norm if isinstance(self.norm2, TokenBatchNorm) else self.norm2
+        order = lambda: _qkv_channel_order(dim, attn.groups, x.device) if attn.channels_first else None
+        if self.local:
+            wq, bq, wp, bp = _prepared(
+                attn, "tokens", x, lambda: _fold_norm(bn1, attn.qkv, order()) + (_dense_weight(attn.proj), attn.proj.bias),
+                deps=_bn_tensors(bn1) + [attn.qkv.weight, attn.qkv.bias, attn.proj.weight, attn.proj.bias])
+            qkv = F.linear(x, wq, bq)
+            t_valid = None if padding is None else (t - padding).to(torch.int32)
+            out = na1d_fused_qkv(qkv.view(n, t, 3, h, dim // h), attn.win_size, attn.left,
+                                 rpb=attn.relative_position_bias, t_valid=t_valid, scale=attn.scale,
+                                 dilation=attn.dilation)
+        else:
+            def build():
+                wq, bq = _dense_weight(attn.qkv), attn.qkv.bias
+                if attn.channels_first:
+                    wq, bq = wq.index_select(0, order()), bq.index_select(0, order())
+                return (wq, bq, _dense_weight(attn.linear_pos), _dense_weight(attn.proj), attn.proj.bias)
+            wq, bq, wl, wp, bp = _prepared(attn, "tokens", x, build, deps=[
+                attn.qkv.weight, attn.qkv.bias, attn.linear_pos.weight, attn.proj.weight, attn.proj.bias])
+            a, b = _bn_affine(bn1)
+            y = torch.addcmul(b + F.linear(pos_emb.to(wl.dtype), wl).float(), x.float(), a).to(wq.dtype)
+            qkv = F.linear(y, wq, bq).view(n, t, 3, h, dim // h).permute(2, 0, 3, 1, 4).contiguous()
+            q, k, v = qkv.view(3, n * h, t, dim // h).unbind(0)
+            t_valid = (t - padding).clamp(0, t).to(torch.int32) if masked else None
+            out = global_attention(q, k, v, h, t_valid, attn.scale)
+            out = out.view(n, h, t, dim // h).transpose(1, 2).reshape(n, t, dim)
+        x = x + F.linear(out, wp, bp)
+        w1, b1, w2, b2 = _prepared(
+            self.mlp, "tokens", x, lambda: _fold_norm(bn2, self.mlp.fc1) + (_dense_weight(self.mlp.fc2), self.mlp.fc2.bias),
+            deps=_bn_tensors(bn2) + [self.mlp.fc1.weight, self.mlp.fc1.bias, self.mlp.fc2.weight, self.mlp.fc2.bias])
+        return x + F.linear(F.gelu(F.linear(x, w1, b1)), w2, b2)
+
 
 class NATFBlock(nn.Module):
     def __init__(self, frames, depth, dim, num_heads, win_size, groups, drop_path, channels_first, dtype, na,
@@ -428,11 +539,24 @@ class NATFBlock(nn.Module):
             for i in range(depth)])
 
     def forward(self, x, padding=None, pos_emb=None, attn_mask_global=None):
+        if (not self.training and not torch.is_grad_enabled() and x.is_cuda
+                and _compute_dtype(x) in (torch.bfloat16, torch.float16) and all(l.tokens_ok() for l in self.blocks)):
+            cf = self.blocks[0].attn.channels_first            # inference: the token-major pipeline
+            pos = pos_emb.transpose(1, 2) if cf and pos_emb is not None else pos_emb
+            y = self.forward_tokens(x.transpose(1, 2).contiguous() if cf else x, padding, pos, attn_mask_global is not None)
+            return y.transpose(1, 2).contiguous() if cf else y
         for layer, ckpt in zip(self.blocks, self.use_checkpoint):
             if ckpt and self.training:      # activation checkpointing re-enters the operator's forward in backward
                 x = torch.utils.checkpoint.checkpoint(layer, x, padding, pos_emb, attn_mask_global, use_reentrant=False)
             else:
                 x = layer(x, padding=padding, pos_emb=pos_emb, attn_mask_global=attn_mask_global)
+        return x
+
+
+    def forward_tokens(self, x, padding=None, pos_emb=None, masked=False):
+        x = x.to(_compute_dtype(x))
+        for layer in self.blocks:
+            x = layer.forward_tokens(x, padding, pos_emb, masked)
         return x
 
 
@@ -446,6 +570,22 @@ class PatchEmbed(nn.Module):
     def forward(self, x):
         x = self.norm(self.proj(x))
         return x if self.channels_first else x.transpose(1, 2)
+
+    def forward_tokens(self, x):
+        """Inference: ``[N, in_chans, frames]`` -> ``[N, T, embed_dim]`` as one matrix product over the patches,
+        with the batch norm folded into it."""
+        conv, bn = self.proj, self.norm
+        n, cin, t = x.shape
+        p, g = conv.kernel_size[0], conv.groups
+        tp = (t - p) // p + 1
+        def build():
+            w = conv.weight.reshape(conv.out_channels, -1).float()           # [cout, (cin/g) * p]
+            w = torch.block_diag(*w.view(g, conv.out_channels // g, -1)) if g > 1 else w
+            a, b = _bn_affine(bn)
+            return w * a.unsqueeze(1), conv.bias.float() * a + b
+        w, b = _prepared(self, "tokens", x, build, deps=[conv.weight, conv.bias] + _bn_tensors(bn))
+        patches = x[:, :, :tp * p].reshape(n, cin, tp, p).permute(0, 2, 1, 3).reshape(n, tp, cin * p)
+        return F.linear(patches.to(w.dtype), w, b)
 
 
 # --------------------------------------------------------------------------- the two model families
@@ -511,6 +651,8 @@ class _NATransformer(nn.Module):
                     mask_global = mask_global.unsqueeze(1)
         if padding is not None:
             padding = padding.to(x.device)
+        if self._tokens_path(x):
+            return self._forward_tokens(x, lens, padding, pos_emb, mask_global is not None)
         outs = []
         if self.channels_first:
             y = None
@@ -527,6 +669,32 @@ class _NATransformer(nn.Module):
             x = torch.cat(outs, dim=-1).transpose(1, 2)
         x = self.proj(self.norm(x))
         return self.fc(self.pool_norm(self.pool(x, lens=lens)))
+
+
+    def _tokens_path(self, x):
+        return (not self.training and not torch.is_grad_enabled() and x.is_cuda
+                and _compute_dtype(x) in (torch.bfloat16, torch.float16)
+                and all(l.tokens_ok() for b in self.blocks for l in b.blocks))
+
+    def _forward_tokens(self, x, lens, padding, pos_emb, masked):
+        """Inference with every activation token-major ``[N, T, C]`` from the patch embedding to the pooling: the
+        same parameters and arithmetic as :meth:`forward`, batch norms folded into the projections behind them,
+        no layout changes between the blocks."""
+        if pos_emb is not None and self.channels_first:
+            pos_emb = pos_emb.transpose(1, 2)
+        outs, y = [], None
+        if self.channels_first:
+            for embed, block in zip(self.patch_embeds, self.blocks):
+                e = embed.forward_tokens(x)
+                y = block.forward_tokens(e if y is None else e + y, padding, pos_emb, masked)
+                outs.append(y)
+        else:
+            y = self.patch_embed.forward_tokens(x)
+            for block in self.blocks:
+                y = block.forward_tokens(y, padding, pos_emb, masked)
+                outs.append(y)
+        h = self.proj.forward_tokens(torch.cat(outs, dim=-1), pre_norm=self.norm)
+        return self.fc(self.pool_norm(self.pool.forward_tokens(h, lens=lens)))
 
 
 class PCF_NATransformer(_NATransformer):

@@ -89,3 +89,41 @@ def test_token_major_projections_equal_the_grouped_convolutions(groups):
     wp = models._dense_weight(layer.proj).unsqueeze(0).expand(n, -1, -1)
     got = torch.baddbmm(layer.proj.bias.view(1, -1, 1), wp, o.transpose(1, 2))
     assert got.is_contiguous() and torch.allclose(got, layer.proj(o.transpose(1, 2)), atol=1e-5)
+
+
+def _random_stats(module, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for name, buf in module.named_buffers():
+            if name.endswith("running_mean"):
+                buf.copy_(torch.randn(buf.shape, generator=g) * 0.3)
+            if name.endswith("running_var"):
+                buf.copy_(torch.rand(buf.shape, generator=g) + 0.5)
+        for p in module.parameters():
+            p.copy_(torch.randn(p.shape, generator=g) * 0.2)
+
+
+@pytest.mark.parametrize("groups", [1, 4])
+def test_token_major_inference_pieces_equal_the_channels_first_modules(groups):
+    """The inference pipeline's restructured pieces (batch norms folded into the neighbouring projections, the
+    pooling's context never concatenated) against the plain modules, in fp32 on the CPU."""
+    g = torch.Generator().manual_seed(3)
+    with torch.no_grad():
+        embed = models.PatchEmbed(8, 16, 2, groups, True).eval()
+        _random_stats(embed, 1)
+        x = torch.randn(3, 8, 21, generator=g)
+        assert torch.allclose(embed.forward_tokens(x), embed(x).transpose(1, 2), atol=1e-5)
+
+        pre, block = models.BatchNorm1d(16).eval(), models.TDNNBlock(16, 24, 1).eval()
+        _random_stats(pre, 2), _random_stats(block, 3)
+        h = torch.randn(3, 16, 10, generator=g)
+        assert torch.allclose(block.forward_tokens(h.transpose(1, 2), pre_norm=pre), block(pre(h)).transpose(1, 2), atol=1e-5)
+        assert torch.allclose(block.forward_tokens(h.transpose(1, 2)), block(h).transpose(1, 2), atol=1e-5)
+
+        pool = models.AttentiveStatisticsPooling(24, attention_channels=8).eval()
+        _random_stats(pool, 4)
+        z = torch.randn(3, 24, 10, generator=g)
+        for lens in (None, torch.tensor([1.0, 0.5, 0.8])):
+            assert torch.allclose(pool.forward_tokens(z.transpose(1, 2).contiguous(), lens), pool(z, lens), atol=1e-5)
+        plain = models.StatisticsPooling()
+        assert torch.allclose(plain.forward_tokens(z.transpose(1, 2).contiguous(), None), plain(z, None))
