@@ -211,3 +211,22 @@ def call_global_backward(dq, dk, dv, q, k, v, out, dout, lse, t_valid, B, H, T, 
                                       _p(t_valid), B, H, T, C, scale, dtype_tag(q.dtype), _p(workspace),
                                       workspace.numel() * workspace.element_size(), _stream(dq))
     check(st, "na1d_global_backward")
+
+
+def call_fused_forward_qkv(out, lse, qkv, rpb, t_valid, W, left, scale):
+    """The strided forward on a contiguous ``[N, T, 3, H, C]`` projection output, ``out`` contiguous
+    ``[N, T, H*C]``: pointers and strides worked out here, without building views (the inference path's
+    per-call overhead).  Returns the status like :func:`call_fused_forward_strided`."""
+    lib = load()
+    N, T, _, H, C = qkv.shape
+    base, step = qkv.data_ptr(), H * C * qkv.element_size()
+    if torch.cuda.current_device() != out.device.index:      # launches go to the device of the tensors
+        with torch.cuda.device(out.device):
+            return call_fused_forward_qkv(out, lse, qkv, rpb, t_valid, W, left, scale)
+    st = lib.na1d_fused_forward_strided(_p(out), _p(lse), base, base + step, base + 2 * step, _p(rpb), _p(t_valid),
+                                        N, H, T, C, W, left, scale, dtype_tag(qkv.dtype),
+                                        (_i64 * 3)(T * 3 * H * C, C, 3 * H * C), (_i64 * 3)(T * H * C, C, H * C),
+                                        _stream(out))
+    if st != UNSUPPORTED:
+        check(st, "na1d_fused_forward_strided")
+    return st

@@ -225,4 +225,18 @@ def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deter
           reference multiplies q by it in 16 bit beforehand).
     Other arguments as in :func:`na1d_fused`.
     """
+    if dilation == 1 and not (torch.is_grad_enabled() and (qkv.requires_grad or (rpb is not None and rpb.requires_grad))):
+        # inference: one library call, no views, no log-sum-exp
+        assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.is_contiguous()
+        N, T, _, H, C = qkv.shape
+        if rpb is not None:
+            rpb = rpb.detach().reshape(H, win_size)
+            if rpb.dtype != torch.float32 or not rpb.is_contiguous():
+                rpb = rpb.to(torch.float32).contiguous()
+        if t_valid is not None:
+            assert t_valid.numel() == N
+            t_valid = t_valid.to(device=qkv.device, dtype=torch.int32).contiguous()
+        out = torch.empty((N, T, H * C), dtype=qkv.dtype, device=qkv.device)
+        if N * T == 0 or _lib.call_fused_forward_qkv(out, None, qkv, rpb, t_valid, win_size, left, float(scale)) == 0:
+            return out
     return _FusedNA1DQKV.apply(qkv, rpb, t_valid, win_size, left, float(scale), bool(deterministic), int(dilation))

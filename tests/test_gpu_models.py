@@ -159,3 +159,22 @@ def test_attention_dropout_in_training_only(na):
     a.float().sum().backward()
     g = drop.blocks[0].blocks[0].attn.qkv.weight.grad
     assert g is not None and torch.isfinite(g).all() and g.abs().sum() > 0
+
+
+@pytest.mark.parametrize("na", ["fused", "fused_qkv"])
+def test_mfa_nat_4x4_inference_with_lengths_fp16(na):
+    """The tokens-first family in inference (fused_qkv: the token-major pipeline with folded batch norms, the
+    global layers masked from the lengths) against the CPU fp32 twin."""
+    cpu = _twin(models.MFA_NATransformer, torch.float16, seed=4).eval()
+    gpu = models.MFA_NATransformer(na=na, dtype=torch.float16)
+    gpu.load_state_dict(cpu.state_dict())
+    gpu = gpu.cuda().eval()
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(5, 80, 260, generator=g)
+    lens = torch.tensor([1.0, 0.7, 0.45, 0.9, 0.62])
+    with torch.no_grad():
+        want = cpu(x, lens)
+        with torch.autocast("cuda", dtype=torch.float16):
+            got = gpu(x.cuda(), lens.cuda())
+    cos = F.cosine_similarity(got.float().cpu(), want, dim=-1)
+    assert cos.min().item() >= 0.999, cos

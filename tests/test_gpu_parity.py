@@ -624,3 +624,19 @@ def test_dropout_rate_zero_is_the_plain_operator_and_bad_rates_are_rejected():
     with pytest.raises(_lib.NA1DError):                               # head_dim > 128 has no dropout kernels
         _lib.call_fused_forward(torch.empty_like(wide), None, wide, wide, wide, None, None, 2, 1, 8, 136, 5, 2, 1.0,
                                 dropout=(0.5, 1))
+
+
+def test_inference_path_of_the_projection_layout_equals_the_autograd_path():
+    """Without gradients na1d_fused_qkv makes one library call on raw pointers; same bits as the autograd path."""
+    N, H, T, C, W, L = 3, 4, 77, 16, 27, 13
+    g = torch.Generator().manual_seed(2)
+    qkv = (torch.randn(N, T, 3, H, C, generator=g) * 0.5).to(torch.bfloat16).cuda()
+    rpb = (torch.randn(1, H, 1, W, generator=g) * 0.3).cuda()
+    tv = torch.tensor([T, 40, 0], dtype=torch.int32).cuda()
+    with torch.no_grad():
+        lean = na1d_fused_qkv(qkv, W, L, rpb=rpb, t_valid=tv, scale=0.25)
+    full = na1d_fused_qkv(qkv.clone().requires_grad_(True), W, L, rpb=rpb, t_valid=tv, scale=0.25)
+    assert lean.shape == (N, T, H * C) and torch.equal(lean, full.detach())
+    with torch.no_grad():                                   # head_dim > 128: falls through to the general path
+        wide = torch.randn(1, 9, 3, 1, 136, generator=g).to(torch.bfloat16).cuda()
+        assert na1d_fused_qkv(wide, 5, 2).shape == (1, 9, 136)
