@@ -196,14 +196,17 @@ int na1d_fused_backward_dropout(void *dq, void *dk, void *dv, float *drpb, const
  * lse [B, T] fp32 (natural log; may be NULL in the forward when no backward follows).  The probabilities are never
  * written to memory.  The backward needs a workspace of na1d_global_backward_workspace_bytes() bytes (one fp32 per
  * row: rowsum(dout * out)) and writes every gradient exactly once, so it is deterministic.
- * C % 8 == 0; C > 128 returns NA1D_ERR_UNSUPPORTED.  Attention dropout (the reference's attn_drop) is not applied:
- * the reference's configurations set it to 0.
+ * C % 8 == 0; C > 128 returns NA1D_ERR_UNSUPPORTED.  p_drop, seed: attention dropout (attn_drop of
+ * models/PCF_NATransformer.py:193,218; 0 in the reference's configurations) by the keep rule stated at
+ * na1d_fused_forward_dropout with the key's row index as the slot j; 0 <= p_drop < 1, 0 switches it off.
  */
 int na1d_global_forward(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
-                        int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, void *stream);
+                        int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, float p_drop, uint64_t seed,
+                        void *stream);
 int na1d_global_backward(void *dq, void *dk, void *dv, const void *q, const void *k, const void *v, const void *out,
                          const void *dout, const float *lse, const int32_t *t_valid, int64_t B, int64_t H, int64_t T,
-                         int64_t C, float scale, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+                         int64_t C, float scale, int dtype, float p_drop, uint64_t seed, void *workspace,
+                         int64_t workspace_bytes, void *stream);
 int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int dtype);
 
 /*

@@ -230,22 +230,24 @@ def global_mask(T, padding=None, dtype=torch.float32):
     return torch.zeros(bad.shape, dtype=dtype).masked_fill(bad, MASK_VALUE)
 
 
-def global_forward(q, k, v, scale, padding=None, num_heads=1):
+def global_forward(q, k, v, scale, padding=None, num_heads=1, keep=None, p_drop=0.0):
     """``softmax(q k^T * scale + mask) v`` per head: returns ``(O, P, LSE)``.
-    models/PCF_NATransformer.py:215-221 (``q * scale`` is applied here to the product instead).
+    models/PCF_NATransformer.py:215-221 (``q * scale`` is applied here to the product instead).  ``keep`` (bool
+    ``[B,T,T]``, e.g. ``dropout_keep(B, T, T, p, seed)``): dropout on the probabilities (:218).
     """
     B, T, _ = q.shape
     z = torch.einsum("btc,buc->btu", q, k) * scale
     m = global_mask(T, padding, dtype=z.dtype)                    # [N or 1, T, T]
     z = (z.view(B // num_heads, num_heads, T, T) + m.unsqueeze(1)).view(B, T, T)
     p = torch.softmax(z, dim=-1)
-    return torch.einsum("btu,buc->btc", p, v), p, torch.logsumexp(z, dim=-1)
+    pd = p if keep is None else p * keep.to(p.dtype) / (1.0 - p_drop)
+    return torch.einsum("btu,buc->btc", pd, v), p, torch.logsumexp(z, dim=-1)
 
 
-def global_backward(q, k, v, do, scale, padding=None, num_heads=1):
+def global_backward(q, k, v, do, scale, padding=None, num_heads=1, keep=None, p_drop=0.0):
     """``(dq, dk, dv)`` by ``torch.autograd`` through :func:`global_forward`."""
     leaves = [x.detach().clone().requires_grad_(True) for x in (q, k, v)]
-    o, _, _ = global_forward(*leaves, scale, padding, num_heads)
+    o, _, _ = global_forward(*leaves, scale, padding, num_heads, keep, p_drop)
     return torch.autograd.grad(o, leaves, do)
 
 

@@ -268,21 +268,27 @@ int na1d_fused_backward_dropout(void *dq, void *dk, void *dv, float *drpb, const
 }
 
 int na1d_global_forward(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
-                        int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, void *stream) {
+                        int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, float p_drop, uint64_t seed,
+                        void *stream) {
     NA1D_CHECK(out, q, k, B, T, C, 1, 0, H, dtype, g);
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
+    g.drop = na1d::make_dropout(p_drop, seed);
     return na1d::mfma::global_fwd(out, lse, q, k, v, t_valid, g, scale, dtype, (hipStream_t)stream);
 }
 
 int na1d_global_backward(void *dq, void *dk, void *dv, const void *q, const void *k, const void *v, const void *out,
                          const void *dout, const float *lse, const int32_t *t_valid, int64_t B, int64_t H, int64_t T,
-                         int64_t C, float scale, int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+                         int64_t C, float scale, int dtype, float p_drop, uint64_t seed, void *workspace,
+                         int64_t workspace_bytes, void *stream) {
     NA1D_CHECK(dq, q, k, B, T, C, 1, 0, H, dtype, g);
     if (!dk || !dv || !v || !out || !dout || !lse || !workspace) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout) || misaligned(workspace))
         return NA1D_ERR_ALIGN;
     if (workspace_bytes < g.B * g.T * (int64_t)sizeof(float)) return NA1D_ERR_SHAPE;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
+    g.drop = na1d::make_dropout(p_drop, seed);
     return na1d::mfma::global_bwd(dq, dk, dv, (float *)workspace, q, k, v, out, dout, lse, t_valid, g, scale, dtype,
                                   (hipStream_t)stream);
 }

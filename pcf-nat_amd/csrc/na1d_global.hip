@@ -52,12 +52,13 @@ struct GlobalArgs {
     uint32_t strips_magic, heads_magic;
     int pitch;                   // bytes per row = 2 * head_dim (packed rows)
     float scale;
+    Dropout drop;                // attention dropout; its window slot is the key's row index
 };
 
 // =============================================================================
 // Forward
 // =============================================================================
-template <class DT, int C>
+template <class DT, int C, bool DROP>
 __global__ void __launch_bounds__(kThreads)
 global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                   const char *__restrict__ k, const char *__restrict__ v, const int32_t *__restrict__ t_valid,
@@ -65,6 +66,7 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     fetch_args_now(out, lse, q, k, v, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic, a.pitch, a.scale);
+    if constexpr (DROP) fetch_args_now(a.drop.threshold, a.drop.seed_lo, a.drop.seed_hi, a.drop.inv_keep);
     constexpr int kStep = region_bytes<C>(kStripTiles);
     extern __shared__ __attribute__((aligned(16))) char smem[];          // 3 * kStep bytes
     LDS_PTR(char) q_lds = (LDS_PTR(char))smem;
@@ -136,6 +138,7 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
         const float alpha = __builtin_amdgcn_exp2f(m - m_new);
         float part = 0.f;
         u32x2 pb[kStripTiles];
+        const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
 #pragma unroll
         for (int kt = 0; kt < kStripTiles; ++kt) {
             float p[4];
@@ -143,6 +146,8 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
             for (int r = 0; r < 4; ++r) {
                 p[r] = __builtin_amdgcn_exp2f(z[kt][r] - m_new);
                 part += p[r];
+                // a dropped probability stays in the sum and leaves O
+                if (DROP && !dropout_keeps(drop_key, 16 * (c0 + kt) + 4 * g + r, a.drop)) p[r] = 0.f;
             }
             pb[kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
         }
@@ -159,7 +164,7 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
         }
     }
     if (qt >= tiles) return;                                // after the last barrier
-    const float inv = __builtin_amdgcn_rcpf(l);
+    const float inv = __builtin_amdgcn_rcpf(l) * (DROP ? a.drop.inv_keep : 1.f);
     u32x2 ow[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
@@ -170,7 +175,7 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
 // =============================================================================
 // Backward, query side: delta = rowsum(dO * O) (written to `delta`) and dQ
 // =============================================================================
-template <class DT, int C>
+template <class DT, int C, bool DROP>
 __global__ void __launch_bounds__(kThreads)
 global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const char *__restrict__ out,
@@ -225,6 +230,8 @@ global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *_
     for (int ct = 0; ct < CT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
     RowOperand<C> qop, gop;
     float dl = 0.f;
+    // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dP = D * (dO . V^T) and delta = rowsum(dO * O) as before.
+    const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
 
     for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
         if (c0) __syncthreads();
@@ -254,7 +261,9 @@ global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *_
                 const int key = 16 * (c0 + kt) + 4 * g + r;
                 const float z = s[r] * scale2 - lse2 + ((key >= tv || row_masked) ? mask2 : 0.f);
                 const float p = key < T ? __builtin_amdgcn_exp2f(z) : 0.f;
-                dsv[r] = p * (dp[r] - dl);
+                float dpr = dp[r];
+                if constexpr (DROP) dpr *= dropout_keeps(drop_key, key, a.drop) ? a.drop.inv_keep : 0.f;
+                dsv[r] = p * (dpr - dl);
             }
             const u32x2 db = {Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
             LDS_PTR(char) blk = k_lds + kt * LL::kTileBytes;
@@ -273,7 +282,7 @@ global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *_
 // =============================================================================
 // Backward, key side: dK and dV
 // =============================================================================
-template <class DT, int C>
+template <class DT, int C, bool DROP>
 __global__ void __launch_bounds__(kThreads)
 global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__restrict__ q, const char *__restrict__ k,
                   const char *__restrict__ v, const char *__restrict__ dout, const float *__restrict__ lse,
@@ -354,7 +363,11 @@ global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__re
                 const int qloc = qi * 16 + 4 * g + r, qrow = 16 * c0 + qloc;
                 const float z = s[r] * scale2 - lse_lds[qloc] * kLog2e + ((col_masked || qrow >= tv) ? mask2 : 0.f);
                 p[r] = qrow < T ? __builtin_amdgcn_exp2f(z) : 0.f;     // rows past the sequence do not exist
-                dsv[r] = p[r] * (dp[r] - del_lds[qloc]);
+                float f = 1.f;             // dropout: dP is masked, and dV takes the probability as the forward used it
+                if constexpr (DROP)
+                    f = dropout_keeps(dropout_row_key((uint64_t)b * T + qrow, a.drop), key, a.drop) ? a.drop.inv_keep : 0.f;
+                dsv[r] = p[r] * (dp[r] * f - del_lds[qloc]);
+                p[r] *= f;
             }
             const u32x2 pb = {Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
             const u32x2 db = {Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
@@ -394,6 +407,7 @@ inline bool global_ok(const Geom &g, GlobalArgs &a, int64_t &items) {
     a.strips_magic = div_magic(a.strips);
     a.heads_magic = div_magic(g.H);
     a.pitch = 2 * g.C;
+    a.drop = g.drop;
     return true;
 }
 
@@ -404,9 +418,10 @@ int launch_global_fwd(void *out, float *lse, const void *q, const void *k, const
     int64_t items;
     if (!global_ok(g, a, items)) return NA1D_ERR_UNSUPPORTED;
     a.scale = scale;
-    if (!allow_lds(global_fwd_kernel<DT, C>, global_lds<C>(3))) return NA1D_ERR_LAUNCH;
-    global_fwd_kernel<DT, C><<<(unsigned)items, kThreads, global_lds<C>(3), s>>>((char *)out, lse, (const char *)q, (const char *)k,
-                                                                 (const char *)v, t_valid, (uint32_t)items, a);
+    auto kern = g.drop.threshold ? global_fwd_kernel<DT, C, true> : global_fwd_kernel<DT, C, false>;
+    if (!allow_lds(kern, global_lds<C>(3))) return NA1D_ERR_LAUNCH;
+    kern<<<(unsigned)items, kThreads, global_lds<C>(3), s>>>((char *)out, lse, (const char *)q, (const char *)k,
+                                                            (const char *)v, t_valid, (uint32_t)items, a);
     return launch_status();
 }
 
@@ -418,14 +433,15 @@ int launch_global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q,
     int64_t items;
     if (!global_ok(g, a, items)) return NA1D_ERR_UNSUPPORTED;
     a.scale = scale;
-    if (!allow_lds(global_dq_kernel<DT, C>, global_lds<C>(5)) || !allow_lds(global_dkv_kernel<DT, C>, global_lds<C>(4)))
-        return NA1D_ERR_LAUNCH;
-    global_dq_kernel<DT, C><<<(unsigned)items, kThreads, global_lds<C>(5), s>>>((char *)dq, delta, (const char *)q, (const char *)k,
-                                                                (const char *)v, (const char *)out, (const char *)dout,
-                                                                lse, t_valid, (uint32_t)items, a);
-    global_dkv_kernel<DT, C><<<(unsigned)items, kThreads, global_lds<C>(4), s>>>((char *)dk, (char *)dv, (const char *)q, (const char *)k,
-                                                                 (const char *)v, (const char *)dout, lse, delta, t_valid,
-                                                                 (uint32_t)items, a);
+    auto dq_kern = g.drop.threshold ? global_dq_kernel<DT, C, true> : global_dq_kernel<DT, C, false>;
+    auto dkv_kern = g.drop.threshold ? global_dkv_kernel<DT, C, true> : global_dkv_kernel<DT, C, false>;
+    if (!allow_lds(dq_kern, global_lds<C>(5)) || !allow_lds(dkv_kern, global_lds<C>(4))) return NA1D_ERR_LAUNCH;
+    dq_kern<<<(unsigned)items, kThreads, global_lds<C>(5), s>>>((char *)dq, delta, (const char *)q, (const char *)k,
+                                                               (const char *)v, (const char *)out, (const char *)dout, lse,
+                                                               t_valid, (uint32_t)items, a);
+    dkv_kern<<<(unsigned)items, kThreads, global_lds<C>(4), s>>>((char *)dk, (char *)dv, (const char *)q, (const char *)k,
+                                                                (const char *)v, (const char *)dout, lse, delta, t_valid,
+                                                                (uint32_t)items, a);
     return launch_status();
 }
 

@@ -67,9 +67,9 @@ def load():
     lib.na1d_fused_backward_dropout.restype = _int
     lib.na1d_fused_backward_dropout.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _f32, _u64, _ptr, _i64, _ptr]
     lib.na1d_global_forward.restype = _int
-    lib.na1d_global_forward.argtypes = [_ptr] * 6 + [_i64] * 4 + [_f32, _int, _ptr]
+    lib.na1d_global_forward.argtypes = [_ptr] * 6 + [_i64] * 4 + [_f32, _int, _f32, _u64, _ptr]
     lib.na1d_global_backward.restype = _int
-    lib.na1d_global_backward.argtypes = [_ptr] * 10 + [_i64] * 4 + [_f32, _int, _ptr, _i64, _ptr]
+    lib.na1d_global_backward.argtypes = [_ptr] * 10 + [_i64] * 4 + [_f32, _int, _f32, _u64, _ptr, _i64, _ptr]
     lib.na1d_global_backward_workspace_bytes.restype = _i64
     lib.na1d_global_backward_workspace_bytes.argtypes = [_i64] * 4 + [_int]
     lib.na1d_profile_events.restype = _int
@@ -186,12 +186,14 @@ def call_fused_backward_strided(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_val
     return st
 
 
-def call_global_forward(out, lse, q, k, v, t_valid, B, H, T, C, scale):
-    """Dense attention over whole sequences; returns the status (``UNSUPPORTED`` for head_dim > 128)."""
+def call_global_forward(out, lse, q, k, v, t_valid, B, H, T, C, scale, dropout=None):
+    """Dense attention over whole sequences; returns the status (``UNSUPPORTED`` for head_dim > 128).
+    ``dropout``: ``None`` or ``(p, seed)``."""
     lib = load()
+    p, seed = dropout or (0.0, 0)
     with torch.cuda.device(out.device):
         st = lib.na1d_global_forward(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(t_valid), B, H, T, C, scale,
-                                     dtype_tag(q.dtype), _stream(out))
+                                     dtype_tag(q.dtype), p, seed, _stream(out))
     if st != UNSUPPORTED:
         check(st, "na1d_global_forward")
     return st
@@ -204,11 +206,12 @@ def global_backward_workspace_bytes(B, H, T, C, dtype) -> int:
     return int(n)
 
 
-def call_global_backward(dq, dk, dv, q, k, v, out, dout, lse, t_valid, B, H, T, C, scale, workspace):
+def call_global_backward(dq, dk, dv, q, k, v, out, dout, lse, t_valid, B, H, T, C, scale, workspace, dropout=None):
     lib = load()
+    p, seed = dropout or (0.0, 0)
     with torch.cuda.device(dq.device):
         st = lib.na1d_global_backward(_p(dq), _p(dk), _p(dv), _p(q), _p(k), _p(v), _p(out), _p(dout), _p(lse),
-                                      _p(t_valid), B, H, T, C, scale, dtype_tag(q.dtype), _p(workspace),
+                                      _p(t_valid), B, H, T, C, scale, dtype_tag(q.dtype), p, seed, _p(workspace),
                                       workspace.numel() * workspace.element_size(), _stream(dq))
     check(st, "na1d_global_backward")
 

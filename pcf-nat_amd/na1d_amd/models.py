@@ -422,11 +422,12 @@ class GlobalAttention(nn.Module):
         q, k, v = _split_heads(self.qkv(x), self.num_heads, self.groups, self.channels_first)
         t, hd = q.shape[1], q.shape[2]
         drop_p = self.attn_drop if self.training else 0.0
-        native = (self.dense == "native" and x.device.type == "cuda" and hd <= 128 and hd % 8 == 0 and drop_p == 0.0
+        native = (self.dense == "native" and x.device.type == "cuda" and hd <= 128 and hd % 8 == 0
                   and q.dtype in (torch.bfloat16, torch.float16) and (attn_mask is None or padding is not None))
         if native:                       # the HIP kernels: no mask or score tensor
             t_valid = None if attn_mask is None else (t - padding).clamp(0, t).to(torch.int32)
-            out = global_attention(q.contiguous(), k.contiguous(), v.contiguous(), self.num_heads, t_valid, self.scale)
+            out = global_attention(q.contiguous(), k.contiguous(), v.contiguous(), self.num_heads, t_valid, self.scale,
+                                   dropout_p=drop_p)
             return self.proj_drop(self.proj(_merge_heads(out, n, self.num_heads, self.channels_first)))
         q, k, v = (z.view(n, self.num_heads, t, hd) for z in (q, k, v))
         if x.device.type == "cuda":      # one library kernel instead of matmul -> mask -> softmax -> matmul

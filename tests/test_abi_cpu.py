@@ -128,15 +128,15 @@ def test_dense_attention_entry_points_validate():
     P, ok = ctypes.c_void_p, ctypes.c_void_p(0x1000)
     f = lib.na1d_global_forward
     args = lambda **kw: [kw.get("o", ok), None, ok, ok, kw.get("v", ok), None, kw.get("B", 4), kw.get("H", 2), 8,
-                         kw.get("C", 16), 1.0, kw.get("dtype", 0), None]
-    assert f(*args(o=None)) == -1 and f(*args(v=None)) == -1
+                         kw.get("C", 16), 1.0, kw.get("dtype", 0), kw.get("p", 0.0), 3, None]
+    assert f(*args(o=None)) == -1 and f(*args(v=None)) == -1 and f(*args(p=1.0)) == -5
     assert f(*args(v=P(0x1004))) == -6
     assert f(*args(C=20)) == -3 and f(*args(dtype=7)) == -2 and f(*args(B=3)) == -5
     assert f(*args(B=0)) == 0                        # nothing to do
     assert f(*args(C=136)) == -8                     # no dense kernel above 128
     b = lib.na1d_global_backward
     bargs = lambda **kw: [ok, ok, ok, ok, ok, ok, kw.get("out", ok), ok, kw.get("lse", ok), None, 4, 2, 8, 16, 1.0, 0,
-                          kw.get("ws", ok), kw.get("wsb", 4 * 8 * 4), None]
+                          0.25, 3, kw.get("ws", ok), kw.get("wsb", 4 * 8 * 4), None]
     assert b(*bargs(out=None)) == -1 and b(*bargs(lse=None)) == -1 and b(*bargs(ws=None)) == -1
     assert b(*bargs(ws=P(0x1008))) == -6
     assert b(*bargs(wsb=4 * 8 * 4 - 1)) == -5        # one fp32 per row is required

@@ -83,3 +83,40 @@ def test_global_attention_rejects_wide_heads():
     q = torch.zeros(1, 4, 136, dtype=torch.bfloat16, device="cuda")
     out = torch.empty_like(q)
     assert _lib.call_global_forward(out, None, q, q, q, None, 1, 1, 4, 136, 1.0) == _lib.UNSUPPORTED
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom", [(2, 2, 37, 32), (1, 3, 130, 64), (2, 1, 100, 24), (1, 2, 300, 16)],
+                         ids=lambda g: "x".join(map(str, g)))
+def test_global_attention_dropout_matches_oracle_with_the_same_mask(geom, dtype):
+    N, H, T, C = geom
+    B, p, seed = N * H, 0.3, 0xFEDC_BA98_7654_3210
+    q, k, v, do = make_inputs(B, T, C, 0, 88, dtype, n=4)
+    scale = C ** -0.5
+    pad = torch.tensor([0, T // 3][:N])
+    t_valid = (T - pad).to(torch.int32).cuda()
+    print("global attention dropout", geom, dtype, flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = global_attention(qd, kd, vd, H, t_valid=t_valid, scale=scale, dropout_p=p, seed=seed)
+    out.backward(do.cuda())
+    keep = O.dropout_keep(B, T, T, p, seed)
+    want_o, _, _ = O.global_forward(q.float(), k.float(), v.float(), scale, pad, H, keep, p)
+    wq, wk, wv = O.global_backward(q.float(), k.float(), v.float(), do.float(), scale, pad, H, keep, p)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float(), want_o) < tol, "O"
+    assert O.rel_l2(qd.grad.float(), wq) < tol, "dQ"
+    assert O.rel_l2(kd.grad.float(), wk) < tol, "dK"
+    assert O.rel_l2(vd.grad.float(), wv) < tol, "dV"
+    again = global_attention(qd.detach(), kd.detach(), vd.detach(), H, t_valid=t_valid, scale=scale, dropout_p=p, seed=seed)
+    assert torch.equal(again, out)
+
+
+def test_global_attention_dropout_mask_is_bit_exact():
+    """One-hot values turn the output into the dropped probability matrix: out[t, u] != 0 exactly where kept."""
+    B, T, C, p, seed = 2, 100, 128, 0.5, 31
+    q = torch.zeros(B, T, C, dtype=torch.float16, device="cuda")
+    v = torch.zeros(B, T, C, dtype=torch.float16)
+    v[:, torch.arange(T), torch.arange(T)] = 1.0
+    out = global_attention(q, q, v.cuda(), 1, scale=1.0, dropout_p=p, seed=seed).cpu()
+    keep = O.dropout_keep(B, T, T, p, seed)
+    assert torch.equal(out[:, :, :T] != 0, keep) and (out[:, :, T:] == 0).all()
