@@ -38,9 +38,10 @@ _library = torch.library.Library(NAMESPACE, "FRAGMENT")   # kept alive for the l
 
 
 def _checked(a: Tensor, b: Tensor, half: int, dtype: torch.dtype, N: int, T: int, C: int, win_size: int, kind: str):
-    """Argument contract shared by the real and the fake kernels; returns the output's (shape, dtype)."""
+    """Argument contract shared by the real and the fake kernels; returns the output's (shape, dtype).  Layout is
+    not part of it: a compiler backend may hand an op a tensor with other strides than the eager program had, so
+    the real kernels pack what is not contiguous, as the reference's ops do (ops_tc240_or_bigger.py:68)."""
     x16, x32 = (a, b)[half], (a, b)[1 - half]
-    torch._check(a.is_contiguous() and b.is_contiguous(), lambda: "NA1D operands must be contiguous")
     torch._check(a.device == b.device, lambda: "NA1D operands must be on one device")
     torch._check(x16.dtype == dtype and tuple(x16.shape) == (N, T, C), lambda: "bad 16-bit operand")
     if kind == "rows":                                    # the other operand is the fp32 score tensor
@@ -58,7 +59,7 @@ def _define_unfused(prefix: str, dtype: torch.dtype, suffix: str):
     def kernel(a, b, N, T, C, win_size, left):
         shape, out_dtype = _checked(a, b, half, dtype, N, T, C, win_size, kind)
         out = torch.empty(shape, dtype=out_dtype, device=a.device)
-        _lib.call_unfused(entry, out, a, b, N, T, C, win_size, left, dtype)
+        _lib.call_unfused(entry, out, a.contiguous(), b.contiguous(), N, T, C, win_size, left, dtype)
         return out
 
     def fake(a, b, N, T, C, win_size, left):
@@ -135,12 +136,11 @@ _library.define("na1d_fused_backward(Tensor dout, Tensor q, Tensor k, Tensor v, 
 
 def _fused_contract(q, k, v, rpb, t_valid, num_heads, win_size):
     torch._check(q.dim() == 3 and q.shape == k.shape == v.shape, lambda: "q, k, v must all be [B, T, C]")
-    torch._check(q.is_contiguous() and k.is_contiguous() and v.is_contiguous(), lambda: "q, k, v must be contiguous")
     torch._check(q.dtype == k.dtype == v.dtype and q.dtype in _DTYPES.values(), lambda: "q, k, v must be bf16 or fp16")
     torch._check(q.shape[0] % num_heads == 0, lambda: "B must be a multiple of num_heads")
     if rpb is not None:
-        torch._check(rpb.dtype == torch.float32 and tuple(rpb.shape) == (num_heads, win_size) and rpb.is_contiguous(),
-                     lambda: "rpb must be contiguous fp32 [num_heads, win_size]")
+        torch._check(rpb.dtype == torch.float32 and tuple(rpb.shape) == (num_heads, win_size),
+                     lambda: "rpb must be fp32 [num_heads, win_size]")
     if t_valid is not None:
         torch._check(t_valid.dtype == torch.int32 and t_valid.numel() == q.shape[0] // num_heads,
                      lambda: "t_valid must be int32 [B / num_heads]")
@@ -149,29 +149,39 @@ def _fused_contract(q, k, v, rpb, t_valid, num_heads, win_size):
 def _fused_forward(q, k, v, rpb, t_valid, num_heads, win_size, left, scale):
     _fused_contract(q, k, v, rpb, t_valid, num_heads, win_size)
     B, T, C = q.shape
+    q, k, v, rpb, t_valid = _packed(q, k, v, rpb, t_valid)
     out = torch.empty_like(q)
     lse = torch.empty((B, T), dtype=torch.float32, device=q.device)
     _lib.call_fused_forward(out, lse, q, k, v, rpb, t_valid, B, num_heads, T, C, win_size, left, scale)
     return out, lse
 
 
+def _packed(*tensors):
+    return tuple(None if t is None else t.contiguous() for t in tensors)
+
+
+def _like(q):
+    return torch.empty(q.shape, dtype=q.dtype, device=q.device)      # contiguous, whatever q's strides
+
+
 def _fused_forward_fake(q, k, v, rpb, t_valid, num_heads, win_size, left, scale):
     _fused_contract(q, k, v, rpb, t_valid, num_heads, win_size)
-    return torch.empty_like(q), torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
+    return _like(q), torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
 
 
 def _fused_backward(dout, q, k, v, out, lse, rpb, t_valid, num_heads, win_size, left, scale, want_drpb):
     B, T, C = q.shape
+    dout, q, k, v, out, lse, rpb, t_valid = _packed(dout, q, k, v, out, lse, rpb, t_valid)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     drpb = torch.zeros((num_heads, win_size) if want_drpb else (0,), dtype=torch.float32, device=q.device)
-    _lib.call_fused_backward(dq, dk, dv, drpb if want_drpb else None, q, k, v, out, dout.contiguous(), lse, rpb,
+    _lib.call_fused_backward(dq, dk, dv, drpb if want_drpb else None, q, k, v, out, dout, lse, rpb,
                              t_valid, B, num_heads, T, C, win_size, left, scale)
     return dq, dk, dv, drpb
 
 
 def _fused_backward_fake(dout, q, k, v, out, lse, rpb, t_valid, num_heads, win_size, left, scale, want_drpb):
     drpb = torch.empty((num_heads, win_size) if want_drpb else (0,), dtype=torch.float32, device=q.device)
-    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), drpb
+    return _like(q), _like(k), _like(v), drpb
 
 
 _library.impl("na1d_fused_forward", _fused_forward, "CUDA")
@@ -221,6 +231,7 @@ _library.define("global_attention_backward(Tensor dout, Tensor q, Tensor k, Tens
 def _dense_forward(q, k, v, t_valid, num_heads, scale):
     _fused_contract(q, k, v, None, t_valid, num_heads, 0)
     B, T, C = q.shape
+    q, k, v, t_valid = _packed(q, k, v, t_valid)
     out = torch.empty_like(q)
     lse = torch.empty((B, T), dtype=torch.float32, device=q.device)
     torch._check(_lib.call_global_forward(out, lse, q, k, v, t_valid, B, num_heads, T, C, scale) == 0,
@@ -230,22 +241,22 @@ def _dense_forward(q, k, v, t_valid, num_heads, scale):
 
 def _dense_forward_fake(q, k, v, t_valid, num_heads, scale):
     _fused_contract(q, k, v, None, t_valid, num_heads, 0)
-    return torch.empty_like(q), torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
+    return _like(q), torch.empty(q.shape[:2], dtype=torch.float32, device=q.device)
 
 
 def _dense_backward(dout, q, k, v, out, lse, t_valid, num_heads, scale):
     B, T, C = q.shape
+    dout, q, k, v, out, lse, t_valid = _packed(dout, q, k, v, out, lse, t_valid)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     if B * T:
         ws = torch.empty(_lib.global_backward_workspace_bytes(B, num_heads, T, C, q.dtype), dtype=torch.uint8,
                          device=q.device)
-        _lib.call_global_backward(dq, dk, dv, q, k, v, out, dout.contiguous(), lse, t_valid, B, num_heads, T, C, scale,
-                                  ws)
+        _lib.call_global_backward(dq, dk, dv, q, k, v, out, dout, lse, t_valid, B, num_heads, T, C, scale, ws)
     return dq, dk, dv
 
 
 def _dense_backward_fake(dout, q, k, v, out, lse, t_valid, num_heads, scale):
-    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    return _like(q), _like(k), _like(v)
 
 
 _library.impl("global_attention_forward", _dense_forward, "CUDA")

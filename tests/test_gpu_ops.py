@@ -94,3 +94,32 @@ def test_dense_attention_op_compiles_and_equals_the_eager_operator():
     x = q.cuda()
     torch.library.opcheck(torch.ops.na_cuda.global_attention_forward.default, (x, x, x, tv, H, 0.2),
                           test_utils=["test_schema", "test_faketensor"])
+
+
+def test_ops_compile_with_the_inductor_backend():
+    """The reference trains under torch.compile (configs/pcf_nat4x4.yaml:28, train_main.py:168-170): the default
+    backend lowers the surrounding torch ops itself and may hand the ops tensors with other strides than eager did,
+    which they pack.  Compiled and eager results agree to rounding, gradients included."""
+    N, H, T, C, W, L, dtype = 2, 4, 60, 16, 27, 13, torch.bfloat16
+    q, k, v, do = make_inputs(N * H, T, C, W, 17, dtype, n=4)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(3)) * 0.3
+
+    def layer(q, k, v, rpb):
+        attn = torch.softmax(ops.ana_qk(q * 0.25, k, W, L) + rpb.repeat(N, 1).unsqueeze(1), dim=-1)
+        return (ops.ana_av(attn, v, W, L) + ops.na1d_fused_op(q, k, v, W, L, rpb=rpb, num_heads=H, scale=0.25)
+                + ops.global_attention_op(q, k, v, H, None, 0.25))
+
+    compiled = torch.compile(layer, backend="inductor", fullgraph=True)
+    ins_e = [t.cuda().requires_grad_(True) for t in (q, k, v, rpb)]
+    ins_c = [t.cuda().requires_grad_(True) for t in (q, k, v, rpb)]
+    oe, oc = layer(*ins_e), compiled(*ins_c)
+    (oe * do.cuda()).float().sum().backward()
+    (oc * do.cuda()).float().sum().backward()
+    assert O.rel_l2(oc.float(), oe.float()) < TOL[dtype]
+    for x, y in zip(ins_c, ins_e):
+        assert O.rel_l2(x.grad.float(), y.grad.float()) < 2 * TOL[dtype]
+    # a transposed view straight into an op: packed inside, same result
+    qt = ins_e[0].detach().transpose(0, 1).contiguous().transpose(0, 1)
+    assert not qt.is_contiguous()
+    assert torch.equal(ops.ana_qk(qt.contiguous(), ins_e[1].detach(), W, L),
+                       torch.ops.na_cuda.bf16_ana_qk_forward(qt, ins_e[1].detach(), N * H, T, C, W, L))
