@@ -11,7 +11,9 @@ models/Pooling.py, models/SoftMaxLoss.py:99-138) in plain torch.nn, built so tha
   ``na="fused_qkv"`` (the same kernels reading q, k, v in place from a token-major qkv projection and
   writing the merged heads directly: no head split / merge copies, no ``q * scale`` pass),
   ``na="unfused"`` (the reference's own chain QK -> +rpb -> +mask -> softmax -> AV
-  through the drop-in Functions), or any callable with the signature of
+  through the drop-in Functions), ``na="fused_op"`` (the fused and the dense operator through their
+  ``torch.library`` registrations, which ``torch.compile`` traces: the reference trains compiled,
+  configs/pcf_nat4x4.yaml:28), or any callable with the signature of
   :func:`na1d_amd.na1d_fused` (tests pass a CPU function here to build a twin).
 
 One class covers both families: PCF-NAT keeps activations channels-first
@@ -367,6 +369,11 @@ class NAttention(nn.Module):
         extra = {} if self.dilation == 1 else {"dilation": self.dilation}
         if callable(self.na):
             out = self.na(q, k, v, w, left, rpb=self.relative_position_bias, t_valid=t_valid, num_heads=h, **extra)
+        elif self.na == "fused_op":
+            from . import ops
+            assert self.dilation == 1 and not dropping, "the registered op covers dilation 1 without dropout"
+            out = ops.na1d_fused_op(q, k, v, w, left, rpb=self.relative_position_bias.view(h, w), t_valid=t_valid,
+                                    num_heads=h, scale=1.0)
         elif self.na in ("fused", "fused_qkv"):              # dropout (PCF :149) happens inside the kernels
             if dropping:
                 extra["dropout_p"] = self.attn_drop
@@ -406,7 +413,7 @@ class GlobalAttention(nn.Module):
 
     def __init__(self, dim, num_heads, groups=1, channels_first=True, dense="native", attn_drop=0.0, proj_drop=0.0):
         super().__init__()
-        assert dense in ("native", "sdpa")
+        assert dense in ("native", "op", "sdpa")
         self.num_heads, self.groups, self.channels_first, self.dense = num_heads, groups, channels_first, dense
         self.attn_drop, self.proj_drop = attn_drop, nn.Dropout(proj_drop)      # PCF :193-195
         self.scale = (dim // num_heads) ** -0.5
@@ -422,12 +429,18 @@ class GlobalAttention(nn.Module):
         q, k, v = _split_heads(self.qkv(x), self.num_heads, self.groups, self.channels_first)
         t, hd = q.shape[1], q.shape[2]
         drop_p = self.attn_drop if self.training else 0.0
-        native = (self.dense == "native" and x.device.type == "cuda" and hd <= 128 and hd % 8 == 0
+        native = (self.dense in ("native", "op") and x.device.type == "cuda" and hd <= 128 and hd % 8 == 0
                   and q.dtype in (torch.bfloat16, torch.float16) and (attn_mask is None or padding is not None))
         if native:                       # the HIP kernels: no mask or score tensor
             t_valid = None if attn_mask is None else (t - padding).clamp(0, t).to(torch.int32)
-            out = global_attention(q.contiguous(), k.contiguous(), v.contiguous(), self.num_heads, t_valid, self.scale,
-                                   dropout_p=drop_p)
+            if self.dense == "op":       # the registered op, for torch.compile
+                from . import ops
+                assert drop_p == 0.0
+                out = ops.global_attention_op(q.contiguous(), k.contiguous(), v.contiguous(), self.num_heads, t_valid,
+                                              self.scale)
+            else:
+                out = global_attention(q.contiguous(), k.contiguous(), v.contiguous(), self.num_heads, t_valid,
+                                       self.scale, dropout_p=drop_p)
             return self.proj_drop(self.proj(_merge_heads(out, n, self.num_heads, self.channels_first)))
         q, k, v = (z.view(n, self.num_heads, t, hd) for z in (q, k, v))
         if x.device.type == "cuda":      # one library kernel instead of matmul -> mask -> softmax -> matmul
@@ -465,7 +478,8 @@ class NATFLayer(nn.Module):
                                    attn_drop, drop)
         else:
             assert dilation == 1
-            self.attn = GlobalAttention(dim, num_heads, groups, channels_first, attn_drop=attn_drop, proj_drop=drop)
+            self.attn = GlobalAttention(dim, num_heads, groups, channels_first, attn_drop=attn_drop, proj_drop=drop,
+                                        dense="op" if na == "fused_op" else "native")
         norm = BatchNorm1d if channels_first else TokenBatchNorm
         self.norm1 = norm(dim)
         self.drop_path = DropPath(drop_path) if drop_path > 0.0 else nn.Identity()
@@ -484,7 +498,7 @@ class NATFLayer(nn.Module):
 
     def tokens_ok(self):
         """Whether :meth:`forward_tokens` serves this layer."""
-        return self.attn.na == "fused_qkv" if self.local else self.attn.dense == "native"
+        return self.attn.na == "fused_qkv" if self.local else self.attn.dense == "native"    # not under torch.compile
 
     def forward_tokens(self, x, padding=None, pos_emb=None, masked=False):
         """The layer in inference on token-major ``x [N, T, C]`` (``pos_emb [1, T, C]``), whatever the layout of

@@ -178,3 +178,28 @@ def test_mfa_nat_4x4_inference_with_lengths_fp16(na):
             got = gpu(x.cuda(), lens.cuda())
     cos = F.cosine_similarity(got.float().cpu(), want, dim=-1)
     assert cos.min().item() >= 0.999, cos
+
+
+def test_model_trains_under_torch_compile():
+    """na="fused_op": the attention layers call the registered ops, so the whole model compiles into one graph
+    (fullgraph) and a training step gives the eager step's loss and gradients."""
+    kw = dict(depths=(2, 2), num_heads=[[16, 4], [16, 16]], win_size=[[27, 0], [27, 27]], groups=(8, 4), frames=120)
+    torch.manual_seed(0)
+    eager = models.PCF_NATransformer(dtype=torch.bfloat16, na="fused", **kw).cuda().train()
+    comp = models.PCF_NATransformer(dtype=torch.bfloat16, na="fused_op", **kw).cuda().train()
+    comp.load_state_dict(eager.state_dict())
+    step = torch.compile(comp, backend="aot_eager", fullgraph=True)
+    x = torch.randn(16, 80, 120, generator=torch.Generator().manual_seed(1)).cuda()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        a, b = eager(x), step(x)
+    assert F.cosine_similarity(a.float(), b.float(), dim=-1).min() > 0.999
+    a.float().pow(2).sum().backward()
+    b.float().pow(2).sum().backward()
+    checked = 0
+    for (name, p), q in zip(eager.named_parameters(), comp.parameters()):
+        if not (name.endswith("weight") or "relative_position_bias" in name):
+            continue                     # a bias in front of a batch norm has an exactly zero gradient: noise both ways
+        if p.grad is not None and p.grad.norm() > 1e-6:
+            assert F.cosine_similarity(p.grad.flatten().float(), q.grad.flatten().float(), dim=0) > 0.97, name
+            checked += 1                 # two bf16 runs through differently decomposed batch norms
+    assert checked > 30
