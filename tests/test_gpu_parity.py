@@ -640,3 +640,41 @@ def test_inference_path_of_the_projection_layout_equals_the_autograd_path():
     with torch.no_grad():                                   # head_dim > 128: falls through to the general path
         wide = torch.randn(1, 9, 3, 1, 136, generator=g).to(torch.bfloat16).cuda()
         assert na1d_fused_qkv(wide, 5, 2).shape == (1, 9, 136)
+
+
+def _guarded(shape, dtype, fill):
+    """A tensor in the middle of a larger allocation whose surroundings hold a sentinel."""
+    n = 1
+    for s in shape:
+        n *= s
+    pad = 4096                                               # elements on each side; keeps 16-byte alignment
+    buf = torch.full((n + 2 * pad,), fill, dtype=dtype, device="cuda")
+    return buf, buf[pad:pad + n].view(shape), pad
+
+
+@pytest.mark.parametrize("geom", [(3, 2, 37, 32, 15, 7), (2, 4, 100, 16, 27, 13), (2, 1, 45, 64, 65, 32), (1, 2, 5, 24, 9, 4),
+                                  (2, 2, 129, 128, 17, 0)], ids=lambda g: "x".join(map(str, g)))
+def test_no_entry_point_writes_outside_its_outputs(geom):
+    """Ragged last tiles, padded head dims and halo rows: every output sits between sentinel bands that must come
+    back untouched (an out-of-bounds store inside the allocation would not fault, it would land there)."""
+    N, H, T, C, W, L = geom
+    B, dtype = N * H, torch.bfloat16
+    q, k, v, do = dev(*make_inputs(B, T, C, W, 61, dtype, n=4))
+    rpb = torch.zeros(H, W, device="cuda")
+    outs = {name: _guarded((B, T, C), dtype, 3.0) for name in ("out", "dq", "dk", "dv", "gout", "gdq", "gdk", "gdv", "av", "kb")}
+    f32 = {name: _guarded(shape, torch.float32, 3.0) for name, shape in
+           (("lse", (B, T)), ("glse", (B, T)), ("attn", (B, T, W)), ("drpb", (H, W)), ("ws", (B, T)))}
+    f32["drpb"][1].zero_()
+    _lib.call_fused_forward(outs["out"][1], f32["lse"][1], q, k, v, rpb, None, B, H, T, C, W, L, 0.3)
+    _lib.call_fused_backward(outs["dq"][1], outs["dk"][1], outs["dv"][1], f32["drpb"][1], q, k, v, outs["out"][1], do,
+                             f32["lse"][1], rpb, None, B, H, T, C, W, L, 0.3)
+    _lib.call_global_forward(outs["gout"][1], f32["glse"][1], q, k, v, None, B, H, T, C, 0.3)
+    _lib.call_global_backward(outs["gdq"][1], outs["gdk"][1], outs["gdv"][1], q, k, v, outs["gout"][1], do, f32["glse"][1],
+                              None, B, H, T, C, 0.3, f32["ws"][1])
+    _lib.call_unfused("na1d_qk_forward", f32["attn"][1], q, k, B, T, C, W, L, dtype)
+    _lib.call_unfused("na1d_av_forward", outs["av"][1], f32["attn"][1], v, B, T, C, W, L, dtype)
+    _lib.call_unfused("na1d_k_backward", outs["kb"][1], f32["attn"][1], q, B, T, C, W, L, dtype)
+    torch.cuda.synchronize()
+    for name, (buf, view, pad) in {**outs, **f32}.items():
+        assert (buf[:pad] == 3.0).all() and (buf[pad + view.numel():] == 3.0).all(), name
+        assert torch.isfinite(view.float()).all(), name
