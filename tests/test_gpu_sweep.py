@@ -2,6 +2,7 @@
 heads, per-sample padding, bias, scale, dropout, both dtypes - against the CPU oracle.  The hand-picked geometries of
 test_gpu_parity.py cover the known edges; this covers the combinations nobody thought of.  Deterministic: the cases
 come from a fixed seed."""
+import os
 import random
 
 import pytest
@@ -13,6 +14,7 @@ from na1d_amd.dense import global_attention
 from _util import TOL, make_inputs, seeded_scores
 
 pytestmark = pytest.mark.gpu
+SCALE = int(os.environ.get("NA1D_SWEEP_SCALE", "1"))      # multiply the number of cases for a longer soak of passing code
 
 
 def _cases(n, seed):
@@ -38,7 +40,7 @@ def _err(got, ref, terms=1):
     return (got - ref).norm().item() / max(ref.norm().item(), 0.05 * (ref.numel() * terms) ** 0.5, 1e-1)
 
 
-@pytest.mark.parametrize("case", _cases(160, 20240607), ids=lambda c: "%d-N%dH%dT%dC%dW%dL%d" % c[:7])
+@pytest.mark.parametrize("case", _cases(160 * SCALE, 20240607), ids=lambda c: "%d-N%dH%dT%dC%dW%dL%d" % c[:7])
 def test_fused_operator_random_geometry(case):
     i, N, H, T, C, W, L, dtype, drop, with_rpb, with_pad, scale = case
     B = N * H
@@ -78,7 +80,7 @@ def test_fused_operator_random_geometry(case):
             assert torch.equal(xd.grad[:, :, j].permute(0, 2, 1, 3).reshape(B, T, C), z.grad)
 
 
-@pytest.mark.parametrize("case", _cases(40, 77), ids=lambda c: "%d-N%dH%dT%dC%d" % c[:5])
+@pytest.mark.parametrize("case", _cases(40 * SCALE, 77), ids=lambda c: "%d-N%dH%dT%dC%d" % c[:5])
 def test_dense_attention_random_geometry(case):
     i, N, H, T, C, _, _, dtype, _, _, with_pad, _ = case
     B = N * H
@@ -98,7 +100,7 @@ def test_dense_attention_random_geometry(case):
     assert O.rel_l2(vd.grad.float(), wv) < tol, "dV"
 
 
-@pytest.mark.parametrize("case", _cases(64, 4242), ids=lambda c: "%d-N%dH%dT%dC%dW%dL%d" % c[:7])
+@pytest.mark.parametrize("case", _cases(64 * SCALE, 4242), ids=lambda c: "%d-N%dH%dT%dC%dW%dL%d" % c[:7])
 def test_unfused_primitives_random_geometry(case):
     """The three drop-in primitives (band QK^T, band . V, inverse-band gather) behind the reference's six calls."""
     i, N, H, T, C, W, L, dtype = case[:8]
