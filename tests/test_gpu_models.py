@@ -203,3 +203,30 @@ def test_model_trains_under_torch_compile():
             assert F.cosine_similarity(p.grad.flatten().float(), q.grad.flatten().float(), dim=0) > 0.97, name
             checked += 1                 # two bf16 runs through differently decomposed batch norms
     assert checked > 30
+
+
+def test_inference_replayed_from_a_captured_graph():
+    """GraphedInference: one capture per input shape, then replays - with lengths as a graph input, eager passes and
+    synchronisations between the replays, and every replay checked against the eager result (some library ops record
+    nodes that do not replay faithfully; the class verifies, and so does this test, on fresh inputs)."""
+    from na1d_amd.graphs import GraphedInference
+    kw = dict(depths=(2, 2), num_heads=[[16, 4], [16, 16]], win_size=[[27, 0], [27, 27]], groups=(8, 4))
+    torch.manual_seed(0)
+    model = models.PCF_NATransformer(dtype=torch.bfloat16, na="fused_qkv", **kw).cuda().eval()
+    _randomise_norm_stats(model, 3)
+    g = torch.Generator().manual_seed(9)
+    x0 = torch.randn(6, 80, 260, generator=g).cuda()
+    lens0 = torch.tensor([1.0, 0.8, 0.5, 0.9, 0.65, 0.72]).cuda()
+    graphed = GraphedInference(model, x0, lens0)
+    for i in range(4):
+        x = torch.randn(6, 80, 260, generator=g).cuda()
+        lens = (0.4 + 0.6 * torch.rand(6, generator=g)).cuda()
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+            want = model(x, lens)
+        torch.cuda.synchronize()
+        got = graphed(x, lens).clone()
+        torch.cuda.synchronize()
+        assert F.cosine_similarity(got.float(), want.float(), dim=-1).min() > 0.9999, i
+        assert (got - want).abs().max() <= 0.05 * want.abs().max()
+    with pytest.raises(AssertionError):
+        graphed(x[:3], lens[:3])                                # another shape needs another capture
