@@ -226,12 +226,54 @@ class StatisticsPooling(nn.Module):
 
 
 # --------------------------------------------------------------------------- attention
+class _TokenLinearFn(torch.autograd.Function):
+    """``x @ w^T + b`` over all tokens with the weight gradient summed in chunks: ``dy^T @ x`` contracts over
+    N*T tokens into a small [out, in] matrix, which the library's matrix product runs on a few dozen workgroups
+    (73 us for 12800 tokens, 256 -> 768 channels); as a batched product over 8 chunks of the tokens plus a sum it
+    takes 27 us."""
+
+    @staticmethod
+    def forward(ctx, x, w, b):
+        dt = _compute_dtype(x)
+        x16, w16 = x.to(dt), w.to(dt)
+        ctx.save_for_backward(x16, w16)
+        ctx.has_bias = b is not None
+        with torch.autocast(x.device.type, enabled=False):
+            return F.linear(x16, w16, None if b is None else b.to(dt))
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        with torch.autocast(dy.device.type, enabled=False):
+            dy = dy.to(x.dtype)
+            x2, dy2 = x.reshape(-1, x.shape[-1]), dy.reshape(-1, dy.shape[-1])
+            m = x2.shape[0]
+            chunks = next((c for c in (8, 4, 2) if m % c == 0 and m // c >= 512), 1)
+            if chunks > 1:
+                dw = torch.bmm(dy2.view(chunks, m // chunks, -1).transpose(1, 2), x2.view(chunks, m // chunks, -1)).sum(0, dtype=torch.float32)
+            else:
+                dw = (dy2.t() @ x2).float()
+            dx = (dy2 @ w).view(x.shape) if ctx.needs_input_grad[0] else None
+            db = dy2.sum(0, dtype=torch.float32) if ctx.has_bias else None
+        return dx, dw, db
+
+
+class TokenLinear(nn.Linear):
+    """nn.Linear on [N, T, C] (same parameters and names); on the GPU in training the backward sums the weight
+    gradient in chunks of tokens."""
+
+    def forward(self, x):
+        if x.is_cuda and torch.is_grad_enabled() and self.weight.requires_grad:
+            return _TokenLinearFn.apply(x, self.weight, self.bias)
+        return super().forward(x)
+
+
 class _Projection(nn.Module):
     """Per-token affine map on either layout: grouped 1x1 conv on [N,C,T] or Linear on [N,T,C]."""
 
     @staticmethod
     def make(cin, cout, bias, groups, channels_first):
-        return Conv1x1(cin, cout, bias=bias, groups=groups) if channels_first else nn.Linear(cin, cout, bias=bias)
+        return Conv1x1(cin, cout, bias=bias, groups=groups) if channels_first else TokenLinear(cin, cout, bias=bias)
 
 
 def _split_heads(x, num_heads, groups, channels_first):
