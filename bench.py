@@ -157,21 +157,24 @@ def model_inference(batch=256, frames=200, steps=10, warmup=3, cpu=True, modes=(
     # small batches are bound by launch overhead, not by the GPU: the same pass replayed from a captured HIP graph
     from na1d_amd.graphs import GraphedInference
     small = {}
-    for nb in (1, 8):
-        xs = xd[:nb].contiguous()
-        graphed = GraphedInference(gpu, xs)
-        def eager():
-            with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
-                return gpu(xs)
-        for name, fn in (("eager_ms", eager), ("graph_ms", lambda: graphed(xs))):
-            for _ in range(3):
-                fn()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(20):
-                fn()
-            torch.cuda.synchronize()
-            small.setdefault("batch_%d" % nb, {})[name] = round((time.perf_counter() - t0) / 20 * 1e3, 3)
+    try:
+        for nb in (1, 8):
+            xs = xd[:nb].contiguous()
+            graphed = GraphedInference(gpu, xs)
+            def eager():
+                with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+                    return gpu(xs)
+            for name, fn in (("eager_ms", eager), ("graph_ms", lambda: graphed(xs))):
+                for _ in range(3):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(20):
+                    fn()
+                torch.cuda.synchronize()
+                small.setdefault("batch_%d" % nb, {})[name] = round((time.perf_counter() - t0) / 20 * 1e3, 3)
+    except Exception as e:      # an extra record: it must not take the headline line down with it
+        small["error"] = "%s: %s" % (type(e).__name__, str(e)[:200])
     res["small_batch_latency"] = small
     if cpu:
         threads = min(os.cpu_count() or 1, 16)
