@@ -331,7 +331,10 @@ def main():
     if not args.no_model:
         del sets
         torch.cuda.empty_cache()
-        line["pcf_nat_4x4_inference"] = model_inference(cpu=not args.no_cpu_baseline)
+        try:
+            line["pcf_nat_4x4_inference"] = model_inference(cpu=not args.no_cpu_baseline)
+        except Exception as e:      # the operator's line above stands on its own
+            line["pcf_nat_4x4_inference"] = {"error": "%s: %s" % (type(e).__name__, str(e)[:300])}
     print(json.dumps(line))
 
 
