@@ -45,8 +45,8 @@ WORKLOADS = {
 # (KiB per dispatch, each scaled by what the same counter reads for a plain copy kernel of known
 # size: x2.0 for FETCH_SIZE, x1.0 for WRITE_SIZE on this machine); None where not measured.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2": int((39087.8 * 2.0 + 57866.5) * 1024),     # fused backward: 80.1 MB read + 59.3 MB written
-    "cfg3": int((19240.9 * 2.0 + 14400.0) * 1024),     # fused forward: 39.4 MB read + 14.7 MB written
+    "cfg2": int((39084.5 * 2.0 + 57865.2) * 1024),     # fused backward: 80.0 MB read + 59.3 MB written
+    "cfg3": int((19241.4 * 2.0 + 14400.0) * 1024),     # fused forward: 39.4 MB read + 14.7 MB written
 }
 
 
