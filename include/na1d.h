@@ -3,9 +3,11 @@
  *
  * C ABI of the shared library.  Every entry point takes raw device pointers,
  * 64-bit sizes, a dtype tag and the HIP stream to launch on; it allocates
- * nothing, keeps no global mutable state, is re-entrant, and returns an int
- * status (NA1D_OK or a negative NA1D_ERR_* code) instead of asserting.  All
- * tensors are dense and contiguous:
+ * nothing and returns an int status (NA1D_OK or a negative NA1D_ERR_* code)
+ * instead of asserting.  The compute entry points are re-entrant and keep no
+ * state between calls, with two stated exceptions at the end of this file:
+ * the profiling hook (a per-thread pair of events) and the kernel-family
+ * switch (one process-wide flag).  All tensors are dense and contiguous:
  *
  *   q, k, v, out, d*  : [B, T, C]  16-bit (bf16 or fp16 by `dtype`), C fastest,
  *                       B = batch * heads (batch major, head minor)
@@ -215,10 +217,21 @@ int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, in
  * recorded by hipExtLaunchKernel: the dispatch's own begin and end, i.e. what a profiler's kernel trace reports,
  * without the gaps between launches that events recorded on the stream include).  Each launch re-records the same
  * pair, so read them (hipEventElapsedTime) or change them between launches.  NULL, NULL switches it off.  With the
- * workspace path of the backward the pair brackets the main kernel, not the small reduction that follows.  Not for
- * use under stream capture.
+ * workspace path of the backward the pair brackets the main kernel, not the small reduction that follows.  While a
+ * pair is set, a launch on a stream that is being captured into a graph is refused with NA1D_ERR_LAUNCH (nothing is
+ * recorded into the graph).
  */
 int na1d_profile_events(void *start, void *stop);
+
+/*
+ * Test hook; no counterpart in the reference.  The library holds two independent implementations of every
+ * operator: the matrix-core kernels and slower generic kernels that also serve the shapes the former do not cover.
+ * na1d_force_generic(1) routes every later call, from any thread, to the generic ones, na1d_force_generic(0) back;
+ * the previous setting is returned.  The initial setting is 1 if the environment holds NA1D_FORCE_GENERIC=1 when
+ * the library is first called, else 0.  The strided entry points, which only the matrix-core kernels serve,
+ * return NA1D_ERR_UNSUPPORTED while it is on.
+ */
+int na1d_force_generic(int on);
 
 /* Bytes of workspace na1d_fused_backward can use for these arguments (0 if it has
  * no use for one, negative status on invalid arguments). */

@@ -1,5 +1,7 @@
-// C ABI of libna1d: argument validation and dispatch.  No torch types, no
-// allocation, no global mutable state; kernels go to the stream that is passed in.
+// C ABI of libna1d: argument validation and dispatch.  No torch types, no allocation; kernels go to the stream
+// that is passed in.  State that outlives a call: the calling thread's profiling events, and the
+// process-wide kernel-family switch.
+#include <atomic>
 #include <cstdlib>
 
 #include "na1d_common.h"
@@ -65,12 +67,17 @@ int check_layout(const int64_t *strides, const Geom &g, na1d::Layout &l) {
         if (st != NA1D_OK) return st > 0 ? NA1D_OK : st; \
     }
 
-// NA1D_FORCE_GENERIC=1 in the environment routes every call to the generic
-// kernels (a second, independent implementation; used by the tests to cross-check).
-inline bool mfma_allowed() {
-    const char *e = std::getenv("NA1D_FORCE_GENERIC");
-    return !(e && e[0] == '1');
+// The generic kernels are a second, independent implementation that the tests cross-check the matrix-core
+// kernels against.  NA1D_FORCE_GENERIC=1 in the environment when the library is first called, or
+// na1d_force_generic(1) at any time, routes every call to them.
+std::atomic<int> &generic_forced() {
+    static std::atomic<int> flag{[] {
+        const char *e = std::getenv("NA1D_FORCE_GENERIC");
+        return (e && e[0] == '1') ? 1 : 0;
+    }()};
+    return flag;
 }
+inline bool mfma_allowed() { return generic_forced().load(std::memory_order_relaxed) == 0; }
 
 // The matrix-core forward: the two/three-block kernel where it covers the window, else the wide-window one.
 int mfma_fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
@@ -299,6 +306,8 @@ int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, in
     if (st < 0) return st;
     return st > 0 ? 0 : g.B * g.T * (int64_t)sizeof(float);
 }
+
+int na1d_force_generic(int on) { return generic_forced().exchange(on ? 1 : 0); }
 
 int na1d_profile_events(void *start, void *stop) {
     na1d::LaunchEvents &ev = na1d::launch_events();

@@ -123,11 +123,17 @@ inline Layout packed_layout(const Geom &g) { return Layout{(int64_t)g.H * g.T * 
 // na1d_profile_events() in na1d.h.  Null, the default, means ordinary launches.
 struct LaunchEvents {
     hipEvent_t start = nullptr, stop = nullptr;
+    bool refused = false;   // a launch was asked to record them on a capturing stream: reported by launch_status()
 };
 LaunchEvents &launch_events();   // thread-local, lives in na1d_api.cpp
 
 // Host-side launch status check.
-inline int launch_status() { return hipGetLastError() == hipSuccess ? NA1D_OK : NA1D_ERR_LAUNCH; }
+inline int launch_status() {
+    LaunchEvents &ev = launch_events();
+    const bool refused = ev.refused;
+    ev.refused = false;
+    return hipGetLastError() == hipSuccess && !refused ? NA1D_OK : NA1D_ERR_LAUNCH;
+}
 
 // ---- generic (any C % 8 == 0, any W <= 80) kernels: na1d_generic.hip -------
 namespace generic {

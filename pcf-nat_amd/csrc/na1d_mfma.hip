@@ -589,7 +589,7 @@ int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const vo
 
 int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype) {
     if (!window_blocks(g)) return 0;
-    switch (g.C) {   // the split does not depend on the dtype
+    switch (padded_width(g.C)) {   // the split does not depend on the dtype
         case 16: return bwd_workspace<BF16, 16>(g);
         case 32: return bwd_workspace<BF16, 32>(g);
         case 64: return bwd_workspace<BF16, 64>(g);

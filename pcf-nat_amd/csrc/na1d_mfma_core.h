@@ -423,11 +423,18 @@ __device__ inline uint32_t xcd_item(uint32_t wg, uint32_t items) {
 // Launch, with the calling thread's profiling events around the kernel if it has set any.
 template <class K, class... Args>
 inline void launch_kernel(K kern, unsigned grid, size_t lds, hipStream_t s, Args... args) {
-    const LaunchEvents &ev = launch_events();
-    if (ev.start || ev.stop)
+    LaunchEvents &ev = launch_events();
+    if (ev.start || ev.stop) {
+        // events recorded by the launch itself do not belong in a captured graph: refuse instead of recording them
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+            ev.refused = true;
+            return;
+        }
         hipExtLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), (uint32_t)lds, s, ev.start, ev.stop, 0, args...);
-    else
+    } else {
         kern<<<grid, kThreads, lds, s>>>(args...);
+    }
 }
 
 // Dynamic LDS above 64 KB has to be allowed per kernel.

@@ -302,11 +302,11 @@ def test_wide_windows_match_oracle(geom, dtype):
     for name, got, want in (("dQ", qd.grad, wq), ("dK", kd.grad, wk), ("dV", vd.grad, wv)):
         assert O.rel_l2(got.float(), want) < tol, name
     assert _err(rd.grad, wr) < tol, "drpb"
-    os.environ["NA1D_FORCE_GENERIC"] = "1"          # the generic kernels are the second opinion
+    _lib.load().na1d_force_generic(1)               # the generic kernels are the second opinion
     try:
         ref, _ = na1d_fused_forward_lse(qd.detach(), kd.detach(), vd.detach(), W, L, rd.detach(), t_valid, H)
     finally:
-        del os.environ["NA1D_FORCE_GENERIC"]
+        _lib.load().na1d_force_generic(0)
     assert O.rel_l2(out.float(), ref.float()) < tol
 
 
@@ -435,7 +435,7 @@ def test_deterministic_rpb_gradient_is_bit_reproducible():
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
 def test_two_kernel_families_agree(dtype):
-    """The matrix-core kernels and the generic kernels are independent implementations; NA1D_FORCE_GENERIC=1
+    """The matrix-core kernels and the generic kernels are independent implementations; na1d_force_generic(1)
     routes the same C-ABI calls to the generic ones."""
     N, H, T, C, W, L = 3, 4, 150, 32, 15, 7
     B = N * H
@@ -455,11 +455,11 @@ def test_two_kernel_families_agree(dtype):
         return [attn, av.float(), ga.float(), o.detach().float(), qd.grad.float(), kd.grad.float(), vd.grad.float(), rd.grad]
 
     fast = run_all()
-    os.environ["NA1D_FORCE_GENERIC"] = "1"
+    assert _lib.load().na1d_force_generic(1) == 0
     try:
         slow = run_all()
     finally:
-        del os.environ["NA1D_FORCE_GENERIC"]
+        assert _lib.load().na1d_force_generic(0) == 1
     assert O.rel_l2(fast[0], slow[0]) < 1e-5
     for a, b in zip(fast[1:], slow[1:]):
         assert O.rel_l2(a, b) < TOL[dtype]
