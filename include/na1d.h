@@ -5,9 +5,10 @@
  * 64-bit sizes, a dtype tag and the HIP stream to launch on; it allocates
  * nothing and returns an int status (NA1D_OK or a negative NA1D_ERR_* code)
  * instead of asserting.  The compute entry points are re-entrant and keep no
- * state between calls, with two stated exceptions at the end of this file:
- * the profiling hook (a per-thread pair of events) and the kernel-family
- * switch (one process-wide flag).  All tensors are dense and contiguous:
+ * state between calls, with three stated exceptions at the end of this file:
+ * the profiling hook (a per-thread pair of events), the kernel-family switch
+ * (one process-wide flag) and na1d_fused_backward_noalloc (a per-GPU scratch
+ * array).  All tensors are dense and contiguous:
  *
  *   q, k, v, out, d*  : [B, T, C]  16-bit (bf16 or fp16 by `dtype`), C fastest,
  *                       B = batch * heads (batch major, head minor)
@@ -43,6 +44,7 @@ extern "C" {
 #define NA1D_ERR_ALIGN       -6   /* a tensor pointer is not 16-byte aligned          */
 #define NA1D_ERR_LAUNCH      -7   /* the HIP runtime rejected the launch              */
 #define NA1D_ERR_UNSUPPORTED -8   /* valid arguments that no built kernel covers      */
+#define NA1D_ERR_TOO_LARGE   -9   /* the problem needs more than the static scratch   */
 
 #define NA1D_MAX_WINDOW 80
 
@@ -237,6 +239,31 @@ int na1d_force_generic(int on);
  * no use for one, negative status on invalid arguments). */
 int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
                                             int dtype);
+
+/*
+ * na1d_fused_backward with a deterministic d rpb and no workspace argument.  It has no counterpart in the
+ * reference; it is for callers that cannot allocate device memory and cannot bring a workspace either: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The per-workgroup partial sums
+ * of d rpb, which na1d_fused_backward puts into the caller's workspace, go into a scratch array of
+ * NA1D_NOALLOC_SCRATCH_BYTES that is part of the library's device code (each GPU the library runs on holds its own
+ * copy until the process ends); the same second kernel folds them in a fixed order.  The call allocates nothing
+ * (no hipMalloc / hipFree, no allocating library routine).  Results are bit-identical to na1d_fused_backward given
+ * a workspace of na1d_fused_backward_workspace_bytes() bytes.
+ *
+ * Limits: the shape must be one the workspace path covers (head_dim <= 128, W <= 32 with at most 16 keys on
+ * either side; otherwise NA1D_ERR_UNSUPPORTED), and na1d_fused_backward_workspace_bytes() for it must not exceed
+ * NA1D_NOALLOC_SCRATCH_BYTES (32768 workgroups), otherwise NA1D_ERR_TOO_LARGE.  All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (different streams or threads) race on it; calls on one
+ * stream are ordered and safe.  The array needs no clearing between calls: a call writes every entry it reads.
+ * The device that owns `stream` must be the current device.
+ */
+#define NA1D_NOALLOC_SCRATCH_BYTES (4 * 1024 * 1024)
+int na1d_fused_backward_noalloc(void *dq, void *dk, void *dv, float *drpb,
+                                const void *q, const void *k, const void *v,
+                                const void *out, const void *dout, const float *lse,
+                                const float *rpb, const int32_t *t_valid,
+                                int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
+                                float scale, int dtype, void *stream);
 
 #ifdef __cplusplus
 }

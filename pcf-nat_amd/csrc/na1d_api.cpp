@@ -1,6 +1,6 @@
 // C ABI of libna1d: argument validation and dispatch.  No torch types, no allocation; kernels go to the stream
-// that is passed in.  State that outlives a call: the calling thread's profiling events, and the
-// process-wide kernel-family switch.
+// that is passed in.  State that outlives a call: the calling thread's profiling events, the process-wide
+// kernel-family switch, and the per-GPU scratch array of na1d_fused_backward_noalloc (na1d_mfma.hip).
 #include <atomic>
 #include <cstdlib>
 
@@ -128,6 +128,7 @@ const char *na1d_status_string(int status) {
         case NA1D_ERR_ALIGN: return "tensor pointers must be 16-byte aligned";
         case NA1D_ERR_LAUNCH: return "HIP rejected the kernel launch";
         case NA1D_ERR_UNSUPPORTED: return "no kernel built for these arguments";
+        case NA1D_ERR_TOO_LARGE: return "the problem needs more scratch than NA1D_NOALLOC_SCRATCH_BYTES";
         default: return "unknown status";
     }
 }
@@ -298,6 +299,25 @@ int na1d_global_backward(void *dq, void *dk, void *dv, const void *q, const void
     g.drop = na1d::make_dropout(p_drop, seed);
     return na1d::mfma::global_bwd(dq, dk, dv, (float *)workspace, q, k, v, out, dout, lse, t_valid, g, scale, dtype,
                                   (hipStream_t)stream);
+}
+
+int na1d_fused_backward_noalloc(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
+                                const void *out, const void *dout, const float *lse, const float *rpb,
+                                const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
+                                int64_t left, float scale, int dtype, void *stream) {
+    NA1D_CHECK(dq, q, k, B, T, C, W, left, H, dtype, g);
+    if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
+    if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
+        return NA1D_ERR_ALIGN;
+    const int64_t need = na1d::mfma::fused_bwd_workspace_bytes(g, dtype);
+    if (need <= 0) return NA1D_ERR_UNSUPPORTED;
+    if (need > na1d::mfma::kStaticScratchBytes) return NA1D_ERR_TOO_LARGE;
+    float *scratch = nullptr;
+    const int ss = na1d::mfma::static_scratch(&scratch);
+    if (ss != NA1D_OK) return ss;
+    const na1d::Layout packed = na1d::packed_layout(g);
+    return na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, packed, packed, scale,
+                                 dtype, scratch, need, (hipStream_t)stream);
 }
 
 int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int dtype) {

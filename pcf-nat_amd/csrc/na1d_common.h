@@ -163,6 +163,9 @@ int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const vo
               const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &out_layout, float scale,
               int dtype, float *workspace, int64_t workspace_bytes, hipStream_t s);
 int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype);   // 0 when the shape is not covered
+// Device address, on the current device, of the library's static scratch array (kStaticScratchBytes bytes).
+constexpr int64_t kStaticScratchBytes = NA1D_NOALLOC_SCRATCH_BYTES;
+int static_scratch(float **ptr);
 // wide windows (W up to 80, any split of it): na1d_mfma_wide.hip
 int wide_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
              const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &out_layout, float scale,

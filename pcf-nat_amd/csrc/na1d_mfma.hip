@@ -1,5 +1,7 @@
 // Fused NA1D forward and backward on the matrix cores (gfx950).  Tiling, LDS layout and
 // operand conventions are described at the top of na1d_mfma_core.h.
+#include <mutex>
+
 #include "na1d_mfma_core.h"
 
 namespace na1d {
@@ -599,6 +601,31 @@ int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype) {
     return 0;
 }
 
+// ---- scratch of the entry point that allocates nothing -----------------------------------------------------
+// na1d_fused_backward_noalloc() keeps the d rpb partial sums (one row of kPartialStride floats per workgroup) in
+// this array instead of a caller's workspace.  Every GPU the library runs on holds its own copy at its own
+// address until the process ends.  In host code the name `scratch` is only a handle: the device address comes
+// from hipGetSymbolAddress, once per device with that device current, and that pointer is what kernels get.
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+int static_scratch(float **ptr) {
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *per_device[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return NA1D_ERR_LAUNCH;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!per_device[dev]) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return NA1D_ERR_LAUNCH;
+        }
+        per_device[dev] = p;
+    }
+    *ptr = static_cast<float *>(per_device[dev]);
+    return NA1D_OK;
+}
 
 }  // namespace mfma
 }  // namespace na1d

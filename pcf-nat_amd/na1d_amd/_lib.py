@@ -24,7 +24,7 @@ SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_b
                       "na1d_fused_forward_strided", "na1d_fused_backward_strided", "na1d_profile_events",
                       "na1d_global_forward", "na1d_global_backward", "na1d_global_backward_workspace_bytes",
                       "na1d_fused_forward_dropout", "na1d_fused_backward_dropout",
-                      "na1d_force_generic",
+                      "na1d_fused_backward_noalloc", "na1d_force_generic",
                       "na1d_version", "na1d_status_string")
 UNSUPPORTED = -8
 
@@ -73,6 +73,8 @@ def load():
     lib.na1d_global_backward.argtypes = [_ptr] * 10 + [_i64] * 4 + [_f32, _int, _f32, _u64, _ptr, _i64, _ptr]
     lib.na1d_global_backward_workspace_bytes.restype = _i64
     lib.na1d_global_backward_workspace_bytes.argtypes = [_i64] * 4 + [_int]
+    lib.na1d_fused_backward_noalloc.restype = _int
+    lib.na1d_fused_backward_noalloc.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _ptr]
     lib.na1d_force_generic.restype = _int
     lib.na1d_force_generic.argtypes = [_int]
     lib.na1d_profile_events.restype = _int

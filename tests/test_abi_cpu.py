@@ -31,7 +31,7 @@ def test_library_exports_every_declared_symbol():
 def test_status_strings():
     lib = _lib.load()
     assert lib.na1d_status_string(0) == b"ok"
-    for code in range(-8, 0):
+    for code in range(-9, 0):
         assert len(lib.na1d_status_string(code)) > 3
     assert lib.na1d_status_string(-99) == b"unknown status"
 
