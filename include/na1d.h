@@ -224,6 +224,10 @@ int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, in
  * recorded into the graph).
  */
 int na1d_profile_events(void *start, void *stop);
+/* Name of the last matrix-core kernel that the calling thread launched while a pair of events was set, spelt as a
+ * kernel trace prints it without namespaces and arguments, e.g. "fused_bwd_kernel<FP16, 32, 2, false>"; "" before the
+ * first such launch.  The string lives in thread-local storage and is overwritten by the next such launch. */
+const char *na1d_profile_last_kernel(void);
 
 /*
  * Test hook; no counterpart in the reference.  The library holds two independent implementations of every

@@ -3,7 +3,13 @@
 // the fused forward and the dense forward, and are compared with index loops written out here in double precision
 // (a restatement of the operator's definition that shares nothing with the library or with the Python oracle).
 // Exit status 0 = every check passed.
+//
+// A second mode, `na1d_abi_check copy R W BYTES ITERS`, times a plain streaming copy: each launch reads R tensors
+// of BYTES bytes, combines them and writes W tensors of BYTES bytes, with every buffer rotated over more than the
+// last-level cache.  It is the yardstick a benchmark holds the operator's kernels against: what the memory system
+// gives a kernel of this launch size that does nothing but move the same number of bytes.
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cmath>
 #include <cstdint>
@@ -208,7 +214,91 @@ int run(int N, int H, int T, int C, int W, int L) {
 
 }  // namespace
 
-int main() {
+namespace {
+
+// ---- streaming-copy yardstick -------------------------------------------------------------------------------
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kCopyThreads = 256, kCopyPerThread = 4;      // 16 KB per workgroup and tensor
+template <int NR, int NW>
+__global__ void __launch_bounds__(kCopyThreads) copy_kernel(u32x4 *const *__restrict__ bufs, size_t n) {
+    const size_t base = (size_t)blockIdx.x * kCopyPerThread * kCopyThreads + threadIdx.x;
+    u32x4 acc[kCopyPerThread];
+#pragma unroll
+    for (int e = 0; e < kCopyPerThread; ++e) acc[e] = u32x4{0, 0, 0, 0};
+#pragma unroll
+    for (int r = 0; r < NR; ++r)
+#pragma unroll
+        for (int e = 0; e < kCopyPerThread; ++e) {
+            const size_t i = base + (size_t)e * kCopyThreads;
+            if (i < n) acc[e] ^= __builtin_nontemporal_load(&bufs[r][i]);      // read once: non-temporal
+        }
+#pragma unroll
+    for (int w = 0; w < NW; ++w)
+#pragma unroll
+        for (int e = 0; e < kCopyPerThread; ++e) {
+            const size_t i = base + (size_t)e * kCopyThreads;
+            acc[e].x += (uint32_t)w;
+            if (i < n) __builtin_nontemporal_store(acc[e], &bufs[NR + w][i]);
+        }
+}
+
+template <int NR, int NW> int time_copy(size_t bytes, int iters) {
+    const size_t n = bytes / 16;
+    const int nb = NR + NW, sets = (int)(700e6 / ((double)nb * (double)bytes)) + 2;
+    std::vector<u32x4 **> dsets;
+    for (int s = 0; s < sets; ++s) {
+        std::vector<u32x4 *> h(nb);
+        for (auto &p : h) {
+            HIP_OK(hipMalloc(&p, bytes));
+            HIP_OK(hipMemset(p, 1, bytes));
+        }
+        u32x4 **d = nullptr;
+        HIP_OK(hipMalloc(&d, nb * sizeof(void *)));
+        HIP_OK(hipMemcpy(d, h.data(), nb * sizeof(void *), hipMemcpyHostToDevice));
+        dsets.push_back(d);
+    }
+    const unsigned grid = (unsigned)((n + kCopyThreads * kCopyPerThread - 1) / (kCopyThreads * kCopyPerThread));
+    for (int it = 0; it < sets + 3; ++it) copy_kernel<NR, NW><<<grid, kCopyThreads>>>(dsets[it % sets], n);
+    HIP_OK(hipDeviceSynchronize());
+    // every launch between its own pair of events recorded by the launch itself: the dispatch's begin and end
+    std::vector<hipEvent_t> ev(2 * (size_t)iters);
+    for (auto &e : ev) HIP_OK(hipEventCreate(&e));
+    for (int it = 0; it < iters; ++it)
+        hipExtLaunchKernelGGL((copy_kernel<NR, NW>), dim3(grid), dim3(kCopyThreads), 0, nullptr, ev[2 * it], ev[2 * it + 1],
+                              0, dsets[it % sets], n);
+    HIP_OK(hipDeviceSynchronize());
+    double total = 0;
+    for (int it = 0; it < iters; ++it) {
+        float ms = 0;
+        HIP_OK(hipEventElapsedTime(&ms, ev[2 * it], ev[2 * it + 1]));
+        total += ms;
+    }
+    const double us = total * 1e3 / iters;
+    std::printf("copy %dR+%dW x %zu bytes, %d launches: copy_us=%.3f GBps=%.1f\n", NR, NW, bytes, iters, us,
+                (double)nb * (double)bytes / us / 1e3);
+    return 0;
+}
+
+int copy_mode(int argc, char **argv) {
+    if (argc != 6) {
+        std::printf("usage: %s copy READS WRITES BYTES ITERS\n", argv[0]);
+        return 64;
+    }
+    const int r = std::atoi(argv[2]), w = std::atoi(argv[3]), iters = std::atoi(argv[5]);
+    const size_t bytes = (size_t)std::atoll(argv[4]) / 16 * 16;
+    if (iters < 1 || iters > 10000 || bytes < 16 || bytes > ((size_t)1 << 31)) return 64;
+    if (r == 3 && w == 1) return time_copy<3, 1>(bytes, iters);
+    if (r == 4 && w == 3) return time_copy<4, 3>(bytes, iters);
+    if (r == 2 && w == 1) return time_copy<2, 1>(bytes, iters);
+    if (r == 1 && w == 1) return time_copy<1, 1>(bytes, iters);
+    std::printf("copy: READS+WRITES must be 1+1, 2+1, 3+1 or 4+3\n");
+    return 64;
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+    if (argc > 1 && std::strcmp(argv[1], "copy") == 0) return copy_mode(argc, argv);
     std::printf("libna1d version %d\n", na1d_version());
     if (run(2, 2, 37, 16, 27, 13) || run(3, 1, 50, 32, 15, 7) || run(1, 2, 20, 64, 33, 16) || run(2, 1, 9, 24, 5, 0)) return 2;
     std::printf(failures ? "%d checks FAILED\n" : "all checks passed\n", failures);

@@ -336,6 +336,8 @@ int na1d_profile_events(void *start, void *stop) {
     return NA1D_OK;
 }
 
+const char *na1d_profile_last_kernel(void) { return na1d::launch_events().kernel; }
+
 int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int64_t W, int64_t left,
                                             int dtype) {
     Geom g;

@@ -124,6 +124,7 @@ inline Layout packed_layout(const Geom &g) { return Layout{(int64_t)g.H * g.T * 
 struct LaunchEvents {
     hipEvent_t start = nullptr, stop = nullptr;
     bool refused = false;   // a launch was asked to record them on a capturing stream: reported by launch_status()
+    char kernel[96] = "";   // name of the last kernel launched with events set (na1d_profile_last_kernel)
 };
 LaunchEvents &launch_events();   // thread-local, lives in na1d_api.cpp
 

@@ -10,16 +10,27 @@ namespace mfma {
 // =============================================================================
 // Fused forward
 // =============================================================================
-template <class DT, int C, int NBV, bool DROP>
+#ifndef NA1D_HG_MT
+#define NA1D_HG_MT 4
+#endif
+constexpr int kGroupTiles = NA1D_HG_MT;      // tiles per strip when heads are staged in groups
+
+// HG heads whose rows lie side by side in memory (a projection's output, head h of a token right behind head h-1)
+// can be staged together: the strip copies then move HG * C channels of a row in one piece - whole 128-byte lines
+// for four heads of 16 channels, where a head alone would ask for quarter lines - into regions laid out as rows of
+// C * HG channels, and every wave computes the tiles of one head (kWaves / HG waves share a head's tiles).
+template <class DT, int C, int NBV, bool DROP, int HG>
 __global__ void __launch_bounds__(kThreads)
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale, uint32_t strips_magic, uint32_t heads_magic, Strides in, Strides outl,
                  int shift, Dropout drop) {
-    using LL = Lds<C>;
+    constexpr int CS = C * HG;                       // channels of a staged row
+    using LL = Lds<CS>;
     constexpr int CT = C / 16;                       // channel tiles of the output
-    constexpr int MT = Strip<C>::kMaxTiles;
+    constexpr int MT = HG > 1 ? kGroupTiles : Strip<CS>::kMaxTiles;
+    static_assert(kWaves % HG == 0, "whole waves per head");
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
@@ -27,41 +38,44 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
     // forward is not short of LDS), Q region of nt tiles
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int key_region = region_bytes<C>(nt + 2);
+    const int key_region = region_bytes<CS>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
     LDS_PTR(char) q_lds = v_lds + key_region;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
-    const uint32_t b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
+    const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H / HG, heads_magic);
+    const int hw = HG > 1 ? wave % HG : 0;           // this wave's head inside the group
+    const uint32_t sample = wi.sample, head0 = wi.head * HG, head = head0 + hw, b = sample * H + head;
     const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
 
     // resources end with the strip (plus its halo), so the fixed-size copy below
     // fetches nothing beyond what this strip needs
-    const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
+    const int64_t in_off = sample * in.sample + head0 * in.head, out_off = sample * outl.sample + head * outl.head;
     const int key_bytes = min(T, 16 * (i1 + 1)) * in.pitch, qry_bytes = min(T, 16 * i1) * in.pitch;
     const Rsrc qs = make_rsrc(q + in_off, qry_bytes), ks = make_rsrc(k + in_off, key_bytes);
     const Rsrc vs = make_rsrc(v + in_off, key_bytes), os = make_rsrc(out + out_off, T * outl.pitch);
     const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
     const bool out_whole_lines = stores_whole_lines(outl.pitch, C, 0);
+    const bool out_grouped = HG > 1 && outl.head == 2 * C && outl.width == 2 * C && outl.pitch >= HG * 2 * C;
 
     // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
     {
-        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
-        if (strips == 1 && (in.pitch == 2 * C || C % 64 == 0)) {      // nobody else reads these rows' lines
-            stage_direct<C, MT + 2, kReadOnce>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
-            stage_direct<C, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadOnce>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+        const int lane_off = direct_lane_offset<CS>(wave, lane, in.pitch, HG * in.width);
+        const bool whole_lines = in.pitch == 2 * C || CS % 64 == 0;
+        if (strips == 1 && whole_lines) {      // nobody else reads these rows' lines
+            stage_direct<CS, MT + 2, kReadOnce>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<CS, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, kReadOnce>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
         } else {
-            stage_direct<C, MT + 2, kReadShared>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
-            if (in.pitch == 2 * C || C % 64 == 0)
-                stage_direct<C, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, kReadShared>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+            if (whole_lines)
+                stage_direct<CS, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
             else
-                stage_direct<C, MT, kReadShared>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadShared>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+                stage_direct<CS, MT, kReadShared>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, kReadShared>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
         }
     }
 
@@ -74,17 +88,17 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     const float scale2 = scale * kLog2e;
 
     // per-lane LDS offsets; key-side regions start 16 rows before the strip
-    RowLane<C> k_lane, q_lane;
-    TrLane<C> v_lane;
-    k_lane.init(16 - shift, lane);
-    q_lane.init(0, lane);
-    v_lane.init(16 - shift, lane);
+    RowLane<C, CS> k_lane, q_lane;
+    TrLane<C, CS> v_lane;
+    k_lane.init(16 - shift, lane, hw * 2 * C);
+    q_lane.init(0, lane, hw * 2 * C);
+    v_lane.init(16 - shift, lane, hw * 2 * C);
 
     wait_direct();
     add_bias<NBV>(win, rpb_raw);
     __syncthreads();
 
-    for (int i = i0 + wave; i < i1; i += kWaves) {
+    for (int i = i0 + wave / HG; i < i1; i += kWaves / HG) {
         const int tile_bytes = (i - i0) * LL::kTileBytes;
         RowOperand<C> qt;
         read_rows<C>(qt, q_lds + tile_bytes, q_lane);
@@ -167,28 +181,74 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
-        store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines, outl.width);
+        if (HG > 1 && out_grouped) {          // into the place of this head's Q tile, which only this wave has read
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)
+                *reinterpret_cast<LDS_PTR(u32x2)>(q_lds + tile_bytes + LL::addr(n, hw * 2 * C + 32 * ct + 8 * g)) = ow[ct];
+        } else {
+            store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines, outl.width);
+        }
         if (g == 0)
             __builtin_amdgcn_raw_buffer_store_b32(
                 __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2), ls, qrow * 4, 0, 0);
     }
+    if (HG > 1 && out_grouped) {
+        // The heads of a group lie side by side in the output too: the strip's output rows, collected in the Q
+        // region, leave as whole lines - the strip copy run backwards, each lane taking the 16-byte unit that sits
+        // at its place in LDS to where it belongs in memory.
+        __syncthreads();
+        constexpr int kRounds = (region_bytes<CS>(MT) / kChunk + kWaves - 1) / kWaves;
+        constexpr int kChunkRows = kChunk / LL::kRowBytes;
+        const Rsrc gs = make_rsrc(out + sample * outl.sample + head0 * outl.head, min(T, 16 * i1) * outl.pitch);
+        const int lane_off = direct_lane_offset<CS>(wave, lane, outl.pitch, HG * outl.width);
+        const int chunks = region_bytes<CS>(i1 - i0) / kChunk;
+#pragma unroll
+        for (int j = 0; j < kRounds; ++j) {
+            const int c = j * kWaves + wave;
+            if (c < chunks) {
+                const u32x4 unit = *reinterpret_cast<LDS_PTR(u32x4)>(q_lds + c * kChunk + lane * 16);
+                __builtin_amdgcn_raw_buffer_store_b128(unit, gs, (16 * i0 + c * kChunkRows) * outl.pitch + lane_off, 0, kStoreAux);
+            }
+        }
+    }
+}
+
+// Heads whose rows lie side by side in memory: 16-channel heads four at a time, 32-channel heads two at a time.
+inline int head_group(const Geom &g, const Layout &in) {
+    const int cw = padded_width(g.C);
+    if (cw != g.C || in.head != g.C || cw > 32) return 1;
+    const int hg = 64 / cw;
+    return (g.H % hg == 0 && in.row >= (int64_t)hg * g.C) ? hg : 1;
+}
+
+template <class DT, int C, int HG>
+int launch_fwd_hg(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
+                  const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &outl, float scale,
+                  hipStream_t s) {
+    const Split sp = make_split(g.B / HG, g.T, HG > 1 ? kGroupTiles : Strip<C>::kMaxTiles);
+    if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
+    const bool two = window_blocks(g) == 2;
+    auto kern = g.drop.threshold
+                    ? (two ? fused_fwd_kernel<DT, C, 2, true, HG> : fused_fwd_kernel<DT, C, 3, true, HG>)
+                    : (two ? fused_fwd_kernel<DT, C, 2, false, HG> : fused_fwd_kernel<DT, C, 3, false, HG>);
+    const size_t lds = (size_t)2 * region_bytes<C * HG>(sp.nt + 2) + region_bytes<C * HG>(sp.nt);
+    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    note_kernel("fused_fwd_kernel", DT::tag, C, two ? 2 : 3, g.drop.threshold != 0, HG);
+    launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
+                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
+                  div_magic(sp.strips), div_magic(g.H / HG), byte_strides(in, g), byte_strides(outl, g), window_shift(g),
+                  g.drop);
+    return launch_status();
 }
 
 template <class DT, int C>
 int launch_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
                const int32_t *t_valid, const Geom &g, const Layout &in, const Layout &outl, float scale, hipStream_t s) {
-    const Split sp = make_split(g.B, g.T, Strip<C>::kMaxTiles);
-    if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
-    const bool two = window_blocks(g) == 2;
-    auto kern = g.drop.threshold ? (two ? fused_fwd_kernel<DT, C, 2, true> : fused_fwd_kernel<DT, C, 3, true>)
-                                 : (two ? fused_fwd_kernel<DT, C, 2, false> : fused_fwd_kernel<DT, C, 3, false>);
-    const size_t lds = (size_t)2 * region_bytes<C>(sp.nt + 2) + region_bytes<C>(sp.nt);
-    if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
-                  rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
-                  div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g),
-                  g.drop);
-    return launch_status();
+    if constexpr (C <= 32) {
+        if (head_group(g, in) > 1)
+            return launch_fwd_hg<DT, C, 64 / C>(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, s);
+    }
+    return launch_fwd_hg<DT, C, 1>(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, s);
 }
 
 int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
@@ -565,6 +625,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
                        (kThreads + (drpb ? kWaves * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    note_kernel("fused_bwd_kernel", DT::tag, C, two ? 2 : 3, g.drop.threshold != 0);
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),

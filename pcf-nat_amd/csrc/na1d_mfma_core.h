@@ -37,6 +37,7 @@
 #pragma once
 
 #include <algorithm>
+#include <cstdio>
 
 #include <hip/hip_ext.h>
 
@@ -192,18 +193,20 @@ template <int C> struct RowOperand {
     u32x4 w32[k32 > 0 ? k32 : 1];
     u32x2 w16[k16 > 0 ? k16 : 1];
 };
-template <int C> struct RowLane {        // this lane's byte offsets for a row operand whose tile starts `row0` rows into a region
+// CS is the width in channels of the rows as they are staged: C, or several heads of C channels side by side, in
+// which case `sub` is the byte offset of this lane's head inside a staged row.
+template <int C, int CS = C> struct RowLane {        // this lane's byte offsets for a row operand whose tile starts `row0` rows into a region
     int off32[RowOperand<C>::k32 > 0 ? RowOperand<C>::k32 : 1];
     int off16;
-    __device__ inline void init(int row0, int lane) {
+    __device__ inline void init(int row0, int lane, int sub = 0) {
         const int g = lane >> 4, n = lane & 15;
 #pragma unroll
-        for (int s = 0; s < RowOperand<C>::k32; ++s) off32[s] = Lds<C>::addr(row0 + n, 64 * s + 16 * g);
-        off16 = Lds<C>::addr(row0 + n, 64 * RowOperand<C>::k32 + 8 * g);
+        for (int s = 0; s < RowOperand<C>::k32; ++s) off32[s] = Lds<CS>::addr(row0 + n, sub + 64 * s + 16 * g);
+        off16 = Lds<CS>::addr(row0 + n, sub + 64 * RowOperand<C>::k32 + 8 * g);
     }
 };
-template <int C>
-__device__ inline void read_rows(RowOperand<C> &o, LDS_PTR(char) tile, const RowLane<C> &l) {
+template <int C, int CS>
+__device__ inline void read_rows(RowOperand<C> &o, LDS_PTR(char) tile, const RowLane<C, CS> &l) {
 #pragma unroll
     for (int s = 0; s < RowOperand<C>::k32; ++s) o.w32[s] = *reinterpret_cast<LDS_PTR(u32x4)>(tile + l.off32[s]);
     if (RowOperand<C>::k16) o.w16[0] = *reinterpret_cast<LDS_PTR(u32x2)>(tile + l.off16);
@@ -219,12 +222,12 @@ __device__ inline f32x4 dot_rows_mma(const RowOperand<C> &a, const RowOperand<C>
 
 // Transposed operand: output lane (n, g) receives tile[row 4g+0..3][chan 16*ct + n];
 // the lane supplies the address of row 4g + (n>>2), byte 32*ct + 8*(n&3).
-template <int C> struct TrLane {
+template <int C, int CS = C> struct TrLane {
     int off[C / 16];
-    __device__ inline void init(int row0, int lane) {
+    __device__ inline void init(int row0, int lane, int sub = 0) {
         const int g = lane >> 4, n = lane & 15;
 #pragma unroll
-        for (int ct = 0; ct < C / 16; ++ct) off[ct] = Lds<C>::addr(row0 + 4 * g + (n >> 2), 32 * ct + 8 * (n & 3));
+        for (int ct = 0; ct < C / 16; ++ct) off[ct] = Lds<CS>::addr(row0 + 4 * g + (n >> 2), sub + 32 * ct + 8 * (n & 3));
     }
 };
 __device__ inline u32x2 read_tr(LDS_PTR(char) p) {
@@ -420,9 +423,23 @@ __device__ inline uint32_t xcd_item(uint32_t wg, uint32_t items) {
     return (wg & 7) * per + (wg >> 3);
 }
 
+// While profiling events are set, the launchers note which kernel they are about to launch, spelt as a profiler's
+// kernel trace prints it without namespaces and arguments, e.g. fused_bwd_kernel<FP16, 32, 2, false>.
+inline void note_kernel(const char *base, int dtype, int C, int nbv, int drop = -1, int hg = 0) {
+    LaunchEvents &ev = launch_events();
+    if (!ev.start && !ev.stop) return;
+    const char *dt = dtype == NA1D_BF16 ? "BF16" : "FP16";
+    if (drop < 0)
+        snprintf(ev.kernel, sizeof ev.kernel, "%s<%s, %d, %d>", base, dt, C, nbv);
+    else if (hg <= 0)
+        snprintf(ev.kernel, sizeof ev.kernel, "%s<%s, %d, %d, %s>", base, dt, C, nbv, drop ? "true" : "false");
+    else
+        snprintf(ev.kernel, sizeof ev.kernel, "%s<%s, %d, %d, %s, %d>", base, dt, C, nbv, drop ? "true" : "false", hg);
+}
+
 // Launch, with the calling thread's profiling events around the kernel if it has set any.
 template <class K, class... Args>
-inline void launch_kernel(K kern, unsigned grid, size_t lds, hipStream_t s, Args... args) {
+inline void launch_kernel_block(K kern, unsigned grid, unsigned block, size_t lds, hipStream_t s, Args... args) {
     LaunchEvents &ev = launch_events();
     if (ev.start || ev.stop) {
         // events recorded by the launch itself do not belong in a captured graph: refuse instead of recording them
@@ -431,10 +448,14 @@ inline void launch_kernel(K kern, unsigned grid, size_t lds, hipStream_t s, Args
             ev.refused = true;
             return;
         }
-        hipExtLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), (uint32_t)lds, s, ev.start, ev.stop, 0, args...);
+        hipExtLaunchKernelGGL(kern, dim3(grid), dim3(block), (uint32_t)lds, s, ev.start, ev.stop, 0, args...);
     } else {
-        kern<<<grid, kThreads, lds, s>>>(args...);
+        kern<<<grid, block, lds, s>>>(args...);
     }
+}
+template <class K, class... Args>
+inline void launch_kernel(K kern, unsigned grid, size_t lds, hipStream_t s, Args... args) {
+    launch_kernel_block(kern, grid, (unsigned)kThreads, lds, s, args...);
 }
 
 // Dynamic LDS above 64 KB has to be allowed per kernel.

@@ -283,7 +283,8 @@ int launch_qk_n(float *attn, const void *a, const void *b, const Geom &g, const 
     auto kern = qk_kernel<DT, C, NBV>;
     const size_t lds = lds_of(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>(attn, (const char *)a, (const char *)b, (uint32_t)sp.items, (int)g.T,
+    note_kernel("qk_kernel", DT::tag, C, NBV);
+    launch_kernel(kern, (unsigned)sp.items, lds, s, attn, (const char *)a, (const char *)b, (uint32_t)sp.items, (int)g.T,
                                                    g.W, g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift, 2 * g.C);
     return launch_status();
 }
@@ -300,7 +301,8 @@ int launch_av_n(void *out, const float *attn, const void *v, const Geom &g, cons
     auto kern = av_kernel<DT, C, NBV>;
     const size_t lds = lds_of(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)v, (uint32_t)sp.items, (int)g.T, g.W,
+    note_kernel("av_kernel", DT::tag, C, NBV);
+    launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, attn, (const char *)v, (uint32_t)sp.items, (int)g.T, g.W,
                                                    g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift, 2 * g.C);
     return launch_status();
 }
@@ -316,7 +318,8 @@ int launch_gather_n(void *out, const float *attn, const void *x, const Geom &g, 
     auto kern = gather_kernel<DT, C, NBV>;
     const size_t lds = lds_of(sp.nt);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)sp.items, kThreads, lds, s>>>((char *)out, attn, (const char *)x, (uint32_t)sp.items, (int)g.T, g.W,
+    note_kernel("gather_kernel", DT::tag, C, NBV);
+    launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, attn, (const char *)x, (uint32_t)sp.items, (int)g.T, g.W,
                                                    g.L, sp.tiles, sp.nt, sp.strips, div_magic(sp.strips), c.shift, 2 * g.C);
     return launch_status();
 }

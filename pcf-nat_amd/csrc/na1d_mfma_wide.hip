@@ -179,6 +179,7 @@ int launch_wide_fwd_n(void *out, float *lse, const void *q, const void *k, const
     const int kt = sp.nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     const size_t lds = (size_t)2 * region_bytes<C>(kt) + region_bytes<C>(sp.nt) + kBiasSlots * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    note_kernel("wide_fwd_kernel", DT::tag, C, NBV, g.drop.threshold != 0);
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
                   div_magic(sp.strips), div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), shift, g.drop);
@@ -492,6 +493,7 @@ int launch_wide_bwd_n(void *dq, void *dk, void *dv, float *drpb, const void *q, 
     auto kern = g.drop.threshold ? wide_bwd_kernel<DT, C, NBV, true> : wide_bwd_kernel<DT, C, NBV, false>;
     const size_t lds = wide_bwd_lds<C>(sp.nt, NBV, w, kv_bytes);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
+    note_kernel("wide_bwd_kernel", DT::tag, C, NBV, g.drop.threshold != 0);
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, kv_bytes, div_magic(sp.strips), div_magic(g.H),

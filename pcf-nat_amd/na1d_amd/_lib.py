@@ -12,7 +12,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libna1d.so")
+LIB_PATH = os.environ.get("NA1D_LIB") or os.path.join(os.path.dirname(_HERE), "lib", "libna1d.so")   # NA1D_LIB: another build
 
 BF16, FP16 = 0, 1
 
@@ -24,7 +24,7 @@ SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_b
                       "na1d_fused_forward_strided", "na1d_fused_backward_strided", "na1d_profile_events",
                       "na1d_global_forward", "na1d_global_backward", "na1d_global_backward_workspace_bytes",
                       "na1d_fused_forward_dropout", "na1d_fused_backward_dropout",
-                      "na1d_fused_backward_noalloc", "na1d_force_generic",
+                      "na1d_fused_backward_noalloc", "na1d_force_generic", "na1d_profile_last_kernel",
                       "na1d_version", "na1d_status_string")
 UNSUPPORTED = -8
 
@@ -79,6 +79,8 @@ def load():
     lib.na1d_force_generic.argtypes = [_int]
     lib.na1d_profile_events.restype = _int
     lib.na1d_profile_events.argtypes = [_ptr, _ptr]
+    lib.na1d_profile_last_kernel.restype = ctypes.c_char_p
+    lib.na1d_profile_last_kernel.argtypes = []
     lib.na1d_version.restype = _int
     lib.na1d_version.argtypes = []
     lib.na1d_status_string.restype = ctypes.c_char_p
