@@ -284,6 +284,10 @@ def config_record(lib, clock, name, layout, steps, warmup, device):
     else:
         which = {"strided": "both", "strided_in": "in", "strided_out": "out"}[layout]
         fwd, bwd = bind_strided(lib, w, make_strided_sets(w, n_sets, device), with_lse=w["bwd"], which=which)
+    shift = int(os.environ.get("NA1D_BENCH_BWD_SHIFT", "0"))
+    if bwd and shift:
+        bwd0 = bwd
+        bwd = lambda i: bwd0(i + shift)
     calls = [fwd] + ([bwd] if bwd else [])
     for i in range(max(warmup, n_sets)):
         for f in calls:

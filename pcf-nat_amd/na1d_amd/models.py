@@ -402,6 +402,8 @@ class NAttention(nn.Module):
         n = x.shape[0]
         t = x.shape[-1] if self.channels_first else x.shape[1]
         h, w, left = self.num_heads, self.win_size, self.left
+        if self.training:       # the reference trains with its constructor-time mask: fixed length, nothing padded (PCF :131-132)
+            padding = None
         t_valid = None if padding is None else (t - padding).to(torch.int32)
         dropping = self.attn_drop > 0.0 and self.training
         if self.na == "fused_qkv" and not dropping:

@@ -230,3 +230,94 @@ def test_inference_replayed_from_a_captured_graph():
         assert (got - want).abs().max() <= 0.05 * want.abs().max()
     with pytest.raises(AssertionError):
         graphed(x[:3], lens[:3])                                # another shape needs another capture
+
+
+def _small_pcf(use_checkpoint, attn_drop, na):
+    torch.manual_seed(11)
+    m = models.PCF_NATransformer(frames=120, embed_dim=64, depths=(2, 2), num_heads=[[4, 1], [4, 4]],
+                                 win_size=[[9, 0], [[8, 3], 9]], groups=[2, 1], proj_channel=96, output_emb_size=32,
+                                 drop_path_rate=0.0, attn_drop=attn_drop, use_checkpoint=use_checkpoint,
+                                 dtype=torch.float16, na=na)
+    return m.cuda().train()
+
+
+@pytest.mark.parametrize("na", ["fused", "fused_qkv", "unfused"])
+@pytest.mark.parametrize("attn_drop", [0.0, 0.2])
+def test_training_with_activation_checkpointing_reenters_the_operator(na, attn_drop):
+    """The reference trains PCF-NAT 6x4 with activation checkpointing (configs/pcf_nat6x4.yaml:62): the layer's
+    forward, and with it the operator's, runs a second time inside backward (models/PCF_NATransformer.py:298-299).
+    One training step with checkpointing must give the loss and the gradients of the same step without it, bit
+    for bit - also with attention dropout, whose mask the recomputation has to draw again identically."""
+    if na == "unfused" and attn_drop > 0:
+        pytest.skip("torch's dropout in the two-call chain draws from the GPU generator; covered by torch itself")
+    x = torch.randn(6, 80, 120, generator=torch.Generator().manual_seed(12)).cuda()
+    results = []
+    for ckpt in (False, True):
+        model = _small_pcf(ckpt, attn_drop, na)
+        torch.manual_seed(13)                       # the seeds of the attention dropout are drawn from here
+        with torch.autocast("cuda", dtype=torch.float16):
+            emb = model(x)
+        loss = emb.float().square().mean()
+        loss.backward()
+        results.append((loss.detach().clone(), [p.grad.detach().clone() for p in model.parameters() if p.grad is not None]))
+    (l0, g0), (l1, g1) = results
+    assert torch.equal(l0, l1) and len(g0) == len(g1) > 10
+    rpb_like = 0
+    for a, b in zip(g0, g1):
+        if a.dim() == 4 and a.shape[0] == 1 and a.shape[2] == 1:       # d rpb is summed with float atomics
+            assert torch.allclose(a, b, rtol=1e-3, atol=1e-6)
+            rpb_like += 1
+        else:
+            assert torch.equal(a, b)
+    assert rpb_like >= 3 and all(g.abs().max() > 0 for g in g0)
+
+
+def test_pcf_nat_6x4_full_batch_agrees_with_the_checked_small_batch():
+    """cfg4 at its full size (64 utterances, 300..2000 frames, padded to the longest): a sample's embedding does
+    not depend on what else is in the batch, so the first and last four samples of the full batch must reproduce
+    an eight-sample batch padded to the same length - the size test_pcf_nat_6x4_variable_length_bf16 holds
+    against the CPU twin."""
+    torch.manual_seed(0)
+    gpu = models.pcf_nat_6x4(na="fused_qkv", dtype=torch.bfloat16).cuda().eval()
+    g = torch.Generator().manual_seed(2)
+    frames = torch.randint(300, 2001, (64,), generator=g)
+    frames[0] = 2000                                   # both batches are padded to 2000 frames
+    tmax = int(frames.max())
+    x = torch.randn(64, 80, tmax, generator=g)
+    for i, f in enumerate(frames):
+        x[i, :, f:] = 0
+    lens = frames.float() / tmax
+    pick = list(range(4)) + list(range(60, 64))
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16):
+        full = gpu(x.cuda(), lens.cuda())
+        small = gpu(x[pick].cuda(), lens[pick].cuda())
+    assert full.shape == (64, 192) and torch.isfinite(full).all()
+    cos = F.cosine_similarity(full[pick].float(), small.float(), dim=-1)
+    assert cos.min().item() >= 0.9999, cos
+
+
+def test_mfa_nat_4x4_full_batch_training_step_agrees_with_the_checked_small_batch():
+    """cfg5 at its full size (batch 128 x 200 frames, fp16 autocast): in training mode batch norm couples the
+    samples, so the full-size step is held against the small one where it can be - in eval mode the embeddings of
+    the first eight samples equal those of an eight-sample batch; in training mode the full step runs, its loss
+    is close to ln(5994) + s * sin(m)-ish for random weights and every gradient is finite and non-zero."""
+    torch.manual_seed(0)
+    gpu = models.MFA_NATransformer(na="fused_qkv", dtype=torch.float16, frames=200).cuda()
+    head = models.ArcMarginSubCenters(192, 5994, m=0.2, s=32.0, subcenters=3).cuda()
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(128, 80, 200, generator=g).cuda()
+    labels = torch.randint(0, 5994, (128,), generator=g).cuda()
+    gpu.eval()
+    with torch.no_grad(), torch.autocast("cuda", dtype=torch.float16):
+        full, small = gpu(x), gpu(x[:8])
+    assert F.cosine_similarity(full[:8].float(), small.float(), dim=-1).min().item() >= 0.9999
+    gpu.train()
+    scaler = torch.amp.GradScaler("cuda", init_scale=1024.0)
+    with torch.autocast("cuda", dtype=torch.float16):
+        emb = gpu(x)
+    loss, _ = head(emb.float(), labels)
+    scaler.scale(loss).backward()
+    assert 6.0 < loss.item() < 30.0
+    grads = [p.grad for p in gpu.parameters() if p.grad is not None]
+    assert len(grads) > 100 and all(torch.isfinite(gr).all() for gr in grads)
+    assert sum(float(gr.abs().max() > 0) for gr in grads) > 0.9 * len(grads)

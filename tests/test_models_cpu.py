@@ -127,3 +127,19 @@ def test_token_major_inference_pieces_equal_the_channels_first_modules(groups):
             assert torch.allclose(pool.forward_tokens(z.transpose(1, 2).contiguous(), lens), pool(z, lens), atol=1e-5)
         plain = models.StatisticsPooling()
         assert torch.allclose(plain.forward_tokens(z.transpose(1, 2).contiguous(), None), plain(z, None))
+
+
+def test_training_mode_uses_the_fixed_length_mask():
+    """The reference's NAttention adds its constructor-time mask (full length, nothing padded) while training and
+    rebuilds the mask from `padding` only in eval mode (models/PCF_NATransformer.py:131-134)."""
+    torch.manual_seed(3)
+    layer = models.NAttention(frames=40, dim=32, num_heads=2, win_size=7, groups=1, channels_first=True,
+                              dtype=torch.float32, na=oracle_na)
+    x = torch.randn(3, 32, 40)
+    pad = torch.tensor([0, 9, 25])
+    layer.train()
+    assert torch.equal(layer(x, padding=pad), layer(x, padding=None))
+    layer.eval()
+    with torch.no_grad():
+        masked, plain = layer(x, padding=pad), layer(x, padding=None)
+    assert torch.equal(masked[0], plain[0]) and not torch.allclose(masked[1:], plain[1:])
