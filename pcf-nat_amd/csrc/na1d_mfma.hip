@@ -25,14 +25,15 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale, uint32_t strips_magic, uint32_t heads_magic, Strides in, Strides outl,
-                 int shift, Dropout drop) {
+                 int shift_arg, Dropout drop) {
+    const int shift = NBV == 3 ? 16 : shift_arg;     // three key blocks always start one tile before the query tile
     constexpr int CS = C * HG;                       // channels of a staged row
     using LL = Lds<CS>;
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = HG > 1 ? kGroupTiles : Strip<CS>::kMaxTiles;
     static_assert(kWaves % HG == 0, "whole waves per head");
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
-                   in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift);
+                   in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
     // dynamic LDS (launch_fwd): K and V regions of nt+2 tiles starting one tile before the strip (row 16*i0 - 16:
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
@@ -45,6 +46,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + region_bytes<CS>(nt)) + (HG > 1 ? wave % HG : 0) * kBiasEntries;   // the bias table of this wave's head
     const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H / HG, heads_magic);
     const int hw = HG > 1 ? wave % HG : 0;           // this wave's head inside the group
     const uint32_t sample = wi.sample, head0 = wi.head * HG, head = head0 + hw, b = sample * H + head;
@@ -79,9 +81,8 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         }
     }
 
-    Window<NBV> win;
-    float rpb_raw[8];
-    make_window<NBV>(win, rpb_raw, rpb ? rpb + head * W : nullptr, W, L, shift, g, n);
+    BiasTable bias_raw;
+    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
@@ -95,7 +96,9 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     v_lane.init(16 - shift, lane, hw * 2 * C);
 
     wait_direct();
-    add_bias<NBV>(win, rpb_raw);
+    write_bias_table(bias_lds, bias_raw, W, lane);
+    Window<NBV> win;
+    read_window<NBV>(win, bias_lds, L, shift, g, n);
     __syncthreads();
 
     for (int i = i0 + wave / HG; i < i1; i += kWaves / HG) {
@@ -231,7 +234,8 @@ int launch_fwd_hg(void *out, float *lse, const void *q, const void *k, const voi
     auto kern = g.drop.threshold
                     ? (two ? fused_fwd_kernel<DT, C, 2, true, HG> : fused_fwd_kernel<DT, C, 3, true, HG>)
                     : (two ? fused_fwd_kernel<DT, C, 2, false, HG> : fused_fwd_kernel<DT, C, 3, false, HG>);
-    const size_t lds = (size_t)2 * region_bytes<C * HG>(sp.nt + 2) + region_bytes<C * HG>(sp.nt);
+    const size_t lds = (size_t)2 * region_bytes<C * HG>(sp.nt + 2) + region_bytes<C * HG>(sp.nt) +
+                       HG * kBiasEntries * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     note_kernel("fused_fwd_kernel", DT::tag, C, two ? 2 : 3, g.drop.threshold != 0, HG);
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
@@ -311,13 +315,14 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
                  int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes, uint32_t strips_magic,
-                 uint32_t heads_magic, Strides in, Strides outl, int shift, Dropout drop) {
+                 uint32_t heads_magic, Strides in, Strides outl, int shift_arg, Dropout drop) {
+    const int shift = NBV == 3 ? 16 : shift_arg;     // three key blocks always start one tile before the query tile
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int MT = StripBwd<C>::kMaxTiles;
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
                    drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width,
-                   outl.sample, outl.head, outl.pitch, outl.width, shift);
+                   outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
     constexpr int kRowsQ = (MT + 2) * 16;
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
@@ -326,7 +331,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // dynamic LDS (see launch_bwd): [K region | V region] of nt+1+NBV tiles each, starting at the first key of
     // query tile i0-1 (row 16*(i0-1) - shift, so that virtual key blocks are whole tiles of the region), reused after
     // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt+2 tiles (rows 16*i0 - 16 ...); lse
-    // of the query-side rows; and - only when d rpb is wanted - 32 slot sums per wave
+    // of the query-side rows; the head's bias table; and - only when d rpb is wanted - 32 slot sums per wave
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = region_bytes<C>(nt + 1 + NBV), qry_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
@@ -335,10 +340,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     LDS_PTR(char) q_lds = k_lds + kv_bytes;
     LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
     LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
-    LDS_PTR(float) rsum = lse_lds + kThreads;      // [kWaves][32] d rpb slot sums per wave
-
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    LDS_PTR(float) bias_lds = lse_lds + kThreads;                           // the head's bias table
+    LDS_PTR(float) rsum = lse_lds + kThreads + kBiasEntries;                // [kWaves][32] d rpb slot sums per wave
     const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
     const uint32_t item = wi.item, b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
     const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
@@ -368,9 +373,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
 
-    Window<NBV> win;
-    float rpb_raw[8];
-    make_window<NBV>(win, rpb_raw, rpb ? rpb + head * W : nullptr, W, L, shift, g, n);
+    BiasTable bias_raw;
+    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
@@ -385,7 +389,9 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     qry_tr.init(0, lane);
 
     wait_direct();
-    add_bias<NBV>(win, rpb_raw);
+    write_bias_table(bias_lds, bias_raw, W, lane);
+    Window<NBV> win;
+    read_window<NBV>(win, bias_lds, L, shift, g, n);
     __syncthreads();
 
     // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
@@ -623,7 +629,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
     const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + 2) * 4 * 512);
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
-                       (kThreads + (drpb ? kWaves * 32 : 0)) * sizeof(float);
+                       (kThreads + kBiasEntries + (drpb ? kWaves * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     note_kernel("fused_bwd_kernel", DT::tag, C, two ? 2 : 3, g.drop.threshold != 0);
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,

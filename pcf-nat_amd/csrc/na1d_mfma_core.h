@@ -124,7 +124,7 @@ template <int C> struct Lds {
     static constexpr int kRowBytes = 2 * C;
     static constexpr int kTileBytes = 16 * kRowBytes;
     static constexpr int kRowsPerPhase = kUnits >= 16 ? 1 : 16 / kUnits;   // rows per 256 bytes
-    __device__ static inline int swz(int row) { return (row / kRowsPerPhase) & (kUnits - 1); }
+    __device__ static inline int swz(int row) { return (int)((uint32_t)row / kRowsPerPhase) & (kUnits - 1); }     // row >= 0
     // byte address of (row, byte-in-row)
     __device__ static inline int addr(int row, int byte) {
         return row * kRowBytes + ((((byte >> 4) ^ swz(row)) << 4) | (byte & 15));
@@ -313,36 +313,38 @@ template <int NBV> struct Window {
     u32x2 keep0, keep2;           // NBV 3: 16-bit lane masks that split packed X into blocks 0 and 2
 };
 
-// Window slots and bias of a lane.  The 8 rpb entries a lane needs are fetched with buffer loads issued
-// BEFORE the strip copies (they are tiny, hit L2, and have long arrived when the copies have; a NULL rpb makes an
-// empty resource, which reads as zeros), so nothing of this is left to do after the workgroup barrier but one
-// multiply-add per slot: bias = raw * log2(e) + (0 inside the band, -inf outside).
-template <int NBV>
-__device__ inline void make_window(Window<NBV> &w, float (&raw)[8], const float *rpb_h, int W, int L, int shift, int g,
-                                   int n) {
+// Window slots and bias of a lane, by way of a small table in LDS.  Every wave writes the table of its head
+// itself - entry i holds the log2-domain bias of window slot j = i - kBiasPad, or -inf where j lies outside
+// [0, W) - with a tiny load issued BEFORE the strip copies (it hits L2; a NULL rpb makes an empty resource, which
+// reads as zeros), and each lane then picks its eight entries with plain LDS reads: no compares, selects or
+// multiply-adds per slot, which for short sequences were a large share of a wave's vector instructions.  Waves
+// that work on the same head share one table: they write the same values, and a wave reads after its own writes.
+constexpr int kBiasPad = 32, kBiasEntries = 64;         // slots -32 .. 31 cover every block's reach (W <= 32)
+struct BiasTable {
+    float raw;
+};
+__device__ inline void load_bias_table(BiasTable &t, const float *rpb_h, int W, int lane) {
     const Rsrc rs = make_rsrc(rpb_h, rpb_h ? W * 4 : 0);
+    t.raw = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, (lane - kBiasPad) * 4, 0, 0));      // outside [0, W): 0
+}
+__device__ inline void write_bias_table(LDS_PTR(float) tab, const BiasTable &t, int W, int lane) {
+    tab[lane] = (uint32_t)(lane - kBiasPad) < (uint32_t)W ? t.raw * kLog2e : kNegInf;
+}
+// The lane's slots out of the wave's own table (written by this wave: program order is enough).
+template <int NBV>
+__device__ inline void read_window(Window<NBV> &w, LDS_PTR(float) tab, int L, int shift, int g, int n) {
+    const int j0 = 4 * g - n + L - shift;               // window slot of register 0 of block 0
     uint32_t m[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-        const int j0 = 4 * g + r - shift - n + L;
-        w.from0[r] = NBV == 2 || j0 >= 0;
-        const int jx = w.from0[r] ? j0 : j0 + 32, jy = j0 + 16;
-        raw[r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, jx * 4, 0, 0));       // outside [0, W): 0
-        raw[4 + r] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, jy * 4, 0, 0));
-        w.bias_x[r] = (jx >= 0 && jx < W) ? 0.f : kNegInf;
-        w.bias_y[r] = (jy >= 0 && jy < W) ? 0.f : kNegInf;
+        w.from0[r] = NBV == 2 || j0 + r >= 0;
+        const int jx = NBV == 3 ? ((j0 + r) & 31) : j0 + r;      // three blocks: block 2's slot where block 0 has none
+        w.bias_x[r] = tab[jx + kBiasPad];
+        w.bias_y[r] = tab[j0 + r + 16 + kBiasPad];
         m[r] = w.from0[r] ? 0xffffu : 0u;
     }
     w.keep0 = u32x2{m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
     w.keep2 = u32x2{~w.keep0.x, ~w.keep0.y};
-}
-template <int NBV>
-__device__ inline void add_bias(Window<NBV> &w, const float (&raw)[8]) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        w.bias_x[r] = __builtin_fmaf(raw[r], kLog2e, w.bias_x[r]);
-        w.bias_y[r] = __builtin_fmaf(raw[4 + r], kLog2e, w.bias_y[r]);
-    }
 }
 
 // Kernel arguments live in memory and the compiler fetches each one next to its
