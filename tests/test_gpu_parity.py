@@ -416,10 +416,11 @@ def test_tensors_beyond_4_gib_are_addressed_with_64_bit_offsets():
     assert torch.equal(a1, attn[B - 1:])
 
 
-def test_deterministic_rpb_gradient_is_bit_reproducible():
+@pytest.mark.parametrize("C,W,L", [(16, 27, 13), (48, 15, 7), (24, 9, 2)], ids=["hd16", "hd48", "hd24"])
+def test_deterministic_rpb_gradient_is_bit_reproducible(C, W, L):
     """With deterministic=True d rpb is folded in a fixed order: two runs give the same bits, and the
-    atomics path agrees with it to fp32 rounding."""
-    N, H, T, C, W, L = 16, 16, 100, 16, 27, 13
+    atomics path agrees with it to fp32 rounding - also for head dims that run at the next kernel width."""
+    N, H, T = 16, 16, 100
     q, k, v, do = make_inputs(N * H, T, C, W, 71, torch.float16, n=4, scale=0.25)
     rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(5)) * 0.3
     grads = []
@@ -431,6 +432,20 @@ def test_deterministic_rpb_gradient_is_bit_reproducible():
     assert all(torch.equal(a, b) for a, b in zip(grads[0], grads[1]))
     assert all(torch.equal(a, b) for a, b in zip(grads[0][1:], grads[2][1:]))       # dq, dk, dv: no atomics at all
     assert torch.allclose(grads[0][0], grads[2][0], rtol=1e-4, atol=1e-4)
+
+
+def test_deterministic_mode_is_refused_where_it_cannot_be_honoured():
+    """Wide windows have no fixed-order reduction of d rpb: asking for one raises instead of falling back to
+    atomics without a word."""
+    N, H, T, C, W, L = 2, 2, 80, 16, 33, 16
+    q, k, v, do = make_inputs(N * H, T, C, W, 72, torch.float16, n=4, scale=0.25)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    rd = (torch.randn(H, W) * 0.3).cuda().requires_grad_(True)
+    out = na1d_fused(qd, kd, vd, W, L, rpb=rd, num_heads=H, deterministic=True)
+    with pytest.raises(_lib.NA1DError, match="deterministic"):
+        out.backward(do.cuda())
+    na1d_fused(qd, kd, vd, W, L, rpb=rd, num_heads=H).backward(do.cuda())          # the default still works
+    assert torch.isfinite(rd.grad).all()
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
