@@ -615,7 +615,7 @@ def main():
     del sets, fwd, bwd, dom
     torch.cuda.empty_cache()
     if not args.no_configs:
-        per_cfg = min(K, 100)
+        per_cfg = max(50, min(K, 100))          # launches per kernel and configuration
         recs, unf = [], []
         try:
             for name in sorted(WORKLOADS):

@@ -16,6 +16,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <algorithm>
 #include <vector>
 
 #include "na1d.h"
@@ -218,33 +219,58 @@ namespace {
 
 // ---- streaming-copy yardstick -------------------------------------------------------------------------------
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-constexpr int kCopyThreads = 256, kCopyPerThread = 4;      // 16 KB per workgroup and tensor
-template <int NR, int NW>
+constexpr int kCopyThreads = 256;
+// EPT 16-byte elements per thread and tensor: 4 KB, 8 KB or 16 KB per workgroup and tensor.  Which is fastest depends
+// on the launch size (small launches want many small workgroups), so the yardstick is the best of the three.
+template <int NR, int NW, int EPT>
 __global__ void __launch_bounds__(kCopyThreads) copy_kernel(u32x4 *const *__restrict__ bufs, size_t n) {
-    const size_t base = (size_t)blockIdx.x * kCopyPerThread * kCopyThreads + threadIdx.x;
-    u32x4 acc[kCopyPerThread];
+    const size_t base = (size_t)blockIdx.x * EPT * kCopyThreads + threadIdx.x;
+    u32x4 acc[EPT];
 #pragma unroll
-    for (int e = 0; e < kCopyPerThread; ++e) acc[e] = u32x4{0, 0, 0, 0};
+    for (int e = 0; e < EPT; ++e) acc[e] = u32x4{0, 0, 0, 0};
 #pragma unroll
     for (int r = 0; r < NR; ++r)
 #pragma unroll
-        for (int e = 0; e < kCopyPerThread; ++e) {
+        for (int e = 0; e < EPT; ++e) {
             const size_t i = base + (size_t)e * kCopyThreads;
             if (i < n) acc[e] ^= __builtin_nontemporal_load(&bufs[r][i]);      // read once: non-temporal
         }
 #pragma unroll
     for (int w = 0; w < NW; ++w)
 #pragma unroll
-        for (int e = 0; e < kCopyPerThread; ++e) {
+        for (int e = 0; e < EPT; ++e) {
             const size_t i = base + (size_t)e * kCopyThreads;
             acc[e].x += (uint32_t)w;
             if (i < n) __builtin_nontemporal_store(acc[e], &bufs[NR + w][i]);
         }
 }
 
+// Average kernel time in us of `iters` launches, every launch between its own pair of events recorded by the launch
+// itself (the dispatch's begin and end), buffers rotated over `sets` sets.
+template <int NR, int NW, int EPT> double time_copy_variant(const std::vector<u32x4 **> &dsets, size_t n, int iters) {
+    const int sets = (int)dsets.size();
+    const unsigned grid = (unsigned)((n + kCopyThreads * EPT - 1) / (kCopyThreads * EPT));
+    for (int it = 0; it < sets + 3; ++it) copy_kernel<NR, NW, EPT><<<grid, kCopyThreads>>>(dsets[it % sets], n);
+    HIP_OK(hipDeviceSynchronize());
+    std::vector<hipEvent_t> ev(2 * (size_t)iters);
+    for (auto &e : ev) HIP_OK(hipEventCreate(&e));
+    for (int it = 0; it < iters; ++it)
+        hipExtLaunchKernelGGL((copy_kernel<NR, NW, EPT>), dim3(grid), dim3(kCopyThreads), 0, nullptr, ev[2 * it],
+                              ev[2 * it + 1], 0, dsets[it % sets], n);
+    HIP_OK(hipDeviceSynchronize());
+    double total = 0;
+    for (int it = 0; it < iters; ++it) {
+        float ms = 0;
+        HIP_OK(hipEventElapsedTime(&ms, ev[2 * it], ev[2 * it + 1]));
+        total += ms;
+    }
+    for (auto &e : ev) HIP_OK(hipEventDestroy(e));
+    return total * 1e3 / iters;
+}
+
 template <int NR, int NW> int time_copy(size_t bytes, int iters) {
     const size_t n = bytes / 16;
-    const int nb = NR + NW, sets = (int)(700e6 / ((double)nb * (double)bytes)) + 2;
+    const int nb = NR + NW, sets = (int)std::min(64.0, 700e6 / ((double)nb * (double)bytes) + 2);
     std::vector<u32x4 **> dsets;
     for (int s = 0; s < sets; ++s) {
         std::vector<u32x4 *> h(nb);
@@ -257,25 +283,11 @@ template <int NR, int NW> int time_copy(size_t bytes, int iters) {
         HIP_OK(hipMemcpy(d, h.data(), nb * sizeof(void *), hipMemcpyHostToDevice));
         dsets.push_back(d);
     }
-    const unsigned grid = (unsigned)((n + kCopyThreads * kCopyPerThread - 1) / (kCopyThreads * kCopyPerThread));
-    for (int it = 0; it < sets + 3; ++it) copy_kernel<NR, NW><<<grid, kCopyThreads>>>(dsets[it % sets], n);
-    HIP_OK(hipDeviceSynchronize());
-    // every launch between its own pair of events recorded by the launch itself: the dispatch's begin and end
-    std::vector<hipEvent_t> ev(2 * (size_t)iters);
-    for (auto &e : ev) HIP_OK(hipEventCreate(&e));
-    for (int it = 0; it < iters; ++it)
-        hipExtLaunchKernelGGL((copy_kernel<NR, NW>), dim3(grid), dim3(kCopyThreads), 0, nullptr, ev[2 * it], ev[2 * it + 1],
-                              0, dsets[it % sets], n);
-    HIP_OK(hipDeviceSynchronize());
-    double total = 0;
-    for (int it = 0; it < iters; ++it) {
-        float ms = 0;
-        HIP_OK(hipEventElapsedTime(&ms, ev[2 * it], ev[2 * it + 1]));
-        total += ms;
-    }
-    const double us = total * 1e3 / iters;
-    std::printf("copy %dR+%dW x %zu bytes, %d launches: copy_us=%.3f GBps=%.1f\n", NR, NW, bytes, iters, us,
-                (double)nb * (double)bytes / us / 1e3);
+    const double t1 = time_copy_variant<NR, NW, 1>(dsets, n, iters), t2 = time_copy_variant<NR, NW, 2>(dsets, n, iters),
+                 t4 = time_copy_variant<NR, NW, 4>(dsets, n, iters);
+    const double us = std::min(t1, std::min(t2, t4));
+    std::printf("copy %dR+%dW x %zu bytes, %d launches: copy_us=%.3f GBps=%.1f (per thread and tensor 1 / 2 / 4 x 16 B: "
+                "%.3f / %.3f / %.3f us)\n", NR, NW, bytes, iters, us, (double)nb * (double)bytes / us / 1e3, t1, t2, t4);
     return 0;
 }
 
