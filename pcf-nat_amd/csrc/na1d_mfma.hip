@@ -95,6 +95,9 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     q_lane.init(0, lane, hw * 2 * C);
     v_lane.init(16 - shift, lane, hw * 2 * C);
 
+    const uint32_t one2 = DT::tag == NA1D_BF16 ? 0x3f803f80u : 0x3c003c00u;
+    const u32x2 ones = {one2, one2};                 // a 16 x 16 block of ones as a matrix operand
+
     wait_direct();
     write_bias_table(bias_lds, bias_raw, W, lane);
     Window<NBV> win;
@@ -139,12 +142,22 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         float m = max3(max3(zx[0], zx[1], zx[2]), max3(zx[3], zy[0], zy[1]), max2(zy[2], zy[3]));
         m = xor_max(m);
 
+        // The row sums that normalise the output come from the matrix core: a product of the rounded probabilities
+        // with a block of ones leaves every lane the sum of its query's row (what the output's numerator was
+        // weighted with, so the row is a weighted mean to the last bit), and saves the vector ALU the adds and the
+        // cross-lane reduction.  The exact fp32 sum is still formed where the log-sum-exp is asked for, and with
+        // dropout, whose row sum is that of the probabilities before any is dropped.
+        constexpr bool kMmaSum = !DROP;
         float px[4], py[4], sum = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             px[r] = __builtin_amdgcn_exp2f(zx[r] - m);
             py[r] = __builtin_amdgcn_exp2f(zy[r] - m);
-            sum += px[r] + py[r];
+        }
+        if (!kMmaSum || lse) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum += px[r] + py[r];
+            sum = xor_sum(sum);
         }
         if constexpr (DROP) {                    // dropped probabilities leave the sum as it is and O without them
             const uint32_t key = dropout_row_key((uint64_t)b * T + qrow, drop);
@@ -158,8 +171,6 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         }
         const u32x2 pkx = {Mma<DT>::pack(px[0], px[1]), Mma<DT>::pack(px[2], px[3])};
         const u32x2 pky = {Mma<DT>::pack(py[0], py[1]), Mma<DT>::pack(py[2], py[3])};
-        sum = xor_sum(sum);
-        const float inv = __builtin_amdgcn_rcpf(sum) * (DROP ? drop.inv_keep : 1.f);
 
         // O^T = sum over blocks of V_blk^T . P^T
         u32x2 pb[NBV];
@@ -170,15 +181,17 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         } else {
             pb[0] = pkx;
         }
-        f32x4 o[CT];
+        f32x4 o[CT], rowsum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
             LDS_PTR(char) blk = v_lds + tile_bytes + vb * LL::kTileBytes;
+            if constexpr (kMmaSum) rowsum = Mma<DT>::k16(ones, pb[vb], rowsum);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr(blk + v_lane.off[ct]), pb[vb], o[ct]);
         }
+        const float inv = __builtin_amdgcn_rcpf(kMmaSum ? rowsum[0] : sum) * (DROP ? drop.inv_keep : 1.f);
 
         // rows past T fall outside the buffer and are dropped by the store
         u32x2 ow[CT];
