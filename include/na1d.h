@@ -179,7 +179,7 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb,
  * and kept probabilities are scaled by 1 / (1 - p_drop); lse is that of the un-dropped softmax.  The mask is a pure
  * function of (seed, b, t, j): the backward recomputes it from the same p_drop and seed, nothing is stored, and the
  * stream differs from torch's (whose mask depends on its launch geometry).  0 <= p_drop < 1.  head_dim > 128
- * returns NA1D_ERR_UNSUPPORTED for p_drop > 0.  All other arguments as in na1d_fused_forward / na1d_fused_backward.
+ * returns NA1D_ERR_UNSUPPORTED for p_drop > 0.  Dilated windows: na1d_fused_forward_strided_dropout.  All other arguments as in na1d_fused_forward / na1d_fused_backward.
  */
 int na1d_fused_forward_dropout(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
                                const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
@@ -189,6 +189,33 @@ int na1d_fused_backward_dropout(void *dq, void *dk, void *dv, float *drpb, const
                                 const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
                                 int64_t left, float scale, int dtype, float p_drop, uint64_t seed, void *workspace,
                                 int64_t workspace_bytes, void *stream);
+
+/*
+ * Attention dropout on strided tensors.  The strided entry points also serve dilated windows: slot j of row t meets
+ * row t + (j - left) * d, so the rows of one residue class t mod d form an undilated problem on every d-th row
+ * (row stride d times the tensor's).  For the dropout mask of such a launch to be the one of the whole operator,
+ * its rows are named by their place in the whole sequence: row t of sequence (n, h) of the launch stands for
+ *     row = (n * H + h) * seq_rows + row_offset + row_stride * t
+ * in the keep rule stated at na1d_fused_forward_dropout (row_stride = d, row_offset = the residue class, seq_rows =
+ * the whole sequence's length; 1, 0, T for an undilated launch).  Replaces nn.Dropout(attn_drop) of the reference's
+ * CPU branch, the only one that runs dilated windows (models/PCF_NATransformer.py:158-170).  Requires
+ * 0 <= row_offset < row_stride and seq_rows >= row_offset + row_stride * (T - 1) + 1.  All other arguments as in
+ * na1d_fused_forward_strided / na1d_fused_backward_strided; NA1D_ERR_UNSUPPORTED when no matrix-core kernel covers the
+ * shape (head_dim > 128): there is no dropout on the generic path.
+ */
+int na1d_fused_forward_strided_dropout(void *out, float *lse, const void *q, const void *k, const void *v,
+                                       const float *rpb, const int32_t *t_valid, int64_t N, int64_t H, int64_t T,
+                                       int64_t C, int64_t W, int64_t left, float scale, int dtype,
+                                       const int64_t *qkv_strides, const int64_t *out_strides, float p_drop,
+                                       uint64_t seed, int64_t row_stride, int64_t row_offset, int64_t seq_rows,
+                                       void *stream);
+int na1d_fused_backward_strided_dropout(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k,
+                                        const void *v, const void *dout, const float *lse, const float *rpb,
+                                        const int32_t *t_valid, int64_t N, int64_t H, int64_t T, int64_t C, int64_t W,
+                                        int64_t left, float scale, int dtype, const int64_t *qkv_strides,
+                                        const int64_t *out_strides, float p_drop, uint64_t seed, int64_t row_stride,
+                                        int64_t row_offset, int64_t seq_rows, void *workspace, int64_t workspace_bytes,
+                                        void *stream);
 
 /*
  * Dense ("global") attention over whole sequences, forward and backward: replaces the body of the reference's

@@ -275,6 +275,53 @@ int na1d_fused_backward_dropout(void *dq, void *dk, void *dv, float *drpb, const
                                     (hipStream_t)stream);
 }
 
+int na1d_fused_forward_strided_dropout(void *out, float *lse, const void *q, const void *k, const void *v,
+                                       const float *rpb, const int32_t *t_valid, int64_t N, int64_t H, int64_t T,
+                                       int64_t C, int64_t W, int64_t left, float scale, int dtype,
+                                       const int64_t *qkv_strides, const int64_t *out_strides, float p_drop,
+                                       uint64_t seed, int64_t row_stride, int64_t row_offset, int64_t seq_rows,
+                                       void *stream) {
+    if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
+    NA1D_CHECK(out, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (!v) return NA1D_ERR_NULL;
+    if (misaligned(v)) return NA1D_ERR_ALIGN;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
+    if (row_stride < 1 || row_offset < 0 || row_offset >= row_stride || seq_rows < row_offset + row_stride * (T - 1) + 1 ||
+        seq_rows > 0x7fffffffLL)
+        return NA1D_ERR_SHAPE;
+    g.drop = na1d::make_dropout(p_drop, seed, (uint32_t)row_stride, (uint32_t)row_offset, (uint32_t)seq_rows);
+    na1d::Layout in, outl;
+    const int ls = check_layout(qkv_strides, g, in), lo = check_layout(out_strides, g, outl);
+    if (ls != NA1D_OK || lo != NA1D_OK) return ls != NA1D_OK ? ls : lo;
+    if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;
+    return mfma_fused_fwd(out, lse, q, k, v, rpb, t_valid, g, in, outl, scale, dtype, (hipStream_t)stream);
+}
+
+int na1d_fused_backward_strided_dropout(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k,
+                                        const void *v, const void *dout, const float *lse, const float *rpb,
+                                        const int32_t *t_valid, int64_t N, int64_t H, int64_t T, int64_t C, int64_t W,
+                                        int64_t left, float scale, int dtype, const int64_t *qkv_strides,
+                                        const int64_t *out_strides, float p_drop, uint64_t seed, int64_t row_stride,
+                                        int64_t row_offset, int64_t seq_rows, void *workspace, int64_t workspace_bytes,
+                                        void *stream) {
+    if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
+    NA1D_CHECK(dq, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (!dk || !dv || !v || !dout || !lse) return NA1D_ERR_NULL;
+    if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(dout)) return NA1D_ERR_ALIGN;
+    if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
+    if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
+    if (row_stride < 1 || row_offset < 0 || row_offset >= row_stride || seq_rows < row_offset + row_stride * (T - 1) + 1 ||
+        seq_rows > 0x7fffffffLL)
+        return NA1D_ERR_SHAPE;
+    g.drop = na1d::make_dropout(p_drop, seed, (uint32_t)row_stride, (uint32_t)row_offset, (uint32_t)seq_rows);
+    na1d::Layout in, outl;
+    const int ls = check_layout(qkv_strides, g, in), lo = check_layout(out_strides, g, outl);
+    if (ls != NA1D_OK || lo != NA1D_OK) return ls != NA1D_OK ? ls : lo;
+    if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;
+    return mfma_fused_bwd(dq, dk, dv, drpb, q, k, v, nullptr, dout, lse, rpb, t_valid, g, in, outl, scale, dtype,
+                          (float *)workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
+}
+
 int na1d_global_forward(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
                         int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, float p_drop, uint64_t seed,
                         void *stream) {

@@ -72,12 +72,18 @@ __device__ inline float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * kL
 //     keep = mix32(key ^ (j * 0x9E3779B9)) >= threshold,                                   threshold = floor(p * 2^32)
 // with mix32 the 32-bit finaliser x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16.
 // Survivors are scaled by 1 / (1 - p).  threshold 0 switches it off.
+// A launch on every d-th row of longer sequences (a dilated window's residue class) names its rows by their place in
+// the whole sequence: row = b * seq_rows + row_offset + row_stride * t for row t of the launch's sequence b.
 struct Dropout {
     uint32_t threshold = 0, seed_lo = 0, seed_hi = 0;
     float inv_keep = 1.f;
+    uint32_t row_stride = 1, row_offset = 0, seq_rows = 0;      // seq_rows 0: the launch's own T
 };
-inline Dropout make_dropout(float p, uint64_t seed) {
+inline Dropout make_dropout(float p, uint64_t seed, uint32_t row_stride = 1, uint32_t row_offset = 0, uint32_t seq_rows = 0) {
     Dropout d;
+    d.row_stride = row_stride;
+    d.row_offset = row_offset;
+    d.seq_rows = seq_rows;
     if (p > 0.f) {
         const double t = (double)p * 4294967296.0;
         d.threshold = t >= 4294967295.0 ? 0xffffffffu : (uint32_t)t;
@@ -97,6 +103,9 @@ __host__ __device__ inline uint32_t mix32(uint32_t x) {
 }
 __host__ __device__ inline uint32_t dropout_row_key(uint64_t row, const Dropout &d) {
     return mix32(mix32((uint32_t)row ^ d.seed_lo) + (uint32_t)(row >> 32) * 0x9E3779B9u + d.seed_hi);
+}
+__host__ __device__ inline uint64_t dropout_row(const Dropout &d, uint64_t b, int T, int t) {
+    return b * (d.seq_rows ? d.seq_rows : (uint32_t)T) + d.row_offset + (uint64_t)d.row_stride * (uint32_t)t;
 }
 __host__ __device__ inline bool dropout_keeps(uint32_t row_key, int slot, const Dropout &d) {
     return mix32(row_key ^ ((uint32_t)slot * 0x9E3779B9u)) >= d.threshold;

@@ -34,7 +34,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     static_assert(kWaves % HG == 0, "whole waves per head");
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
-    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
     // dynamic LDS (launch_fwd): K and V regions of nt+2 tiles starting one tile before the strip (row 16*i0 - 16:
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
     // forward is not short of LDS), Q region of nt tiles
@@ -160,7 +160,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
             sum = xor_sum(sum);
         }
         if constexpr (DROP) {                    // dropped probabilities leave the sum as it is and O without them
-            const uint32_t key = dropout_row_key((uint64_t)b * T + qrow, drop);
+            const uint32_t key = dropout_row_key(dropout_row(drop, b, T, qrow), drop);
             const int j0 = 4 * g - n + L - shift;                    // window slot of register 0 of set X
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -336,7 +336,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
                    drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width,
                    outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
-    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
     constexpr int kRowsQ = (MT + 2) * 16;
     constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
@@ -461,7 +461,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dV takes D*P and dP = D * (dO . V^T).
         float fx[4] = {1.f, 1.f, 1.f, 1.f}, fy[4] = {1.f, 1.f, 1.f, 1.f};
         if constexpr (DROP) {
-            const uint32_t key = dropout_row_key((uint64_t)b * T + qrow, drop);
+            const uint32_t key = dropout_row_key(dropout_row(drop, b, T, qrow), drop);
             const int j0 = 4 * g - n + L - shift;                    // window slot of register 0 of set X
 #pragma unroll
             for (int r = 0; r < 4; ++r) {

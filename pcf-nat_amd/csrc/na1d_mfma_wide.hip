@@ -52,7 +52,7 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
     constexpr int MT = Strip<C>::kMaxTiles;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift);
-    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
     // dynamic LDS (launch_wide_fwd): K and V regions of kt tiles starting sb tiles before the strip, Q region of nt
     // tiles, kBiasSlots bias floats
     const int sb = (shift + 15) >> 4;                        // whole tiles in front of the strip
@@ -134,7 +134,7 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
         m = xor_max(m);
         float sum = 0.f;
         u32x2 pb[NBV];
-        const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, drop) : 0u;
+        const uint32_t drop_key = DROP ? dropout_row_key(dropout_row(drop, b, T, qrow), drop) : 0u;
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
             float p[4];
@@ -245,7 +245,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
                    kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width, outl.sample,
                    outl.head, outl.pitch, outl.width, shift);
-    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep);
+    if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
     const int hb = NBV - 1 - (shift >> 4), ha = (shift + 15) >> 4;
     const int qtiles = nt + hb + ha;                        // query-side tiles, <= kWideQueryTiles
     const int ktiles = qtiles + NBV - 1;                    // key-side tiles: whole virtual blocks
@@ -332,7 +332,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
         const bool edge = s0 < 0 || s0 + 16 * NBV > tv;
         float p[NBV][4], dp[NBV][4], part = 0.f;
         // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dV takes D*P and dP = D * (dO . V^T).
-        const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, drop) : 0u;
+        const uint32_t drop_key = DROP ? dropout_row_key(dropout_row(drop, b, T, qrow), drop) : 0u;
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
             RowOperand<C> kop, vop;

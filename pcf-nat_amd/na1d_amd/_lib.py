@@ -25,6 +25,7 @@ SYMBOLS = _UNFUSED + ("na1d_fused_forward", "na1d_fused_backward", "na1d_fused_b
                       "na1d_global_forward", "na1d_global_backward", "na1d_global_backward_workspace_bytes",
                       "na1d_fused_forward_dropout", "na1d_fused_backward_dropout",
                       "na1d_fused_backward_noalloc", "na1d_force_generic", "na1d_profile_last_kernel",
+                      "na1d_fused_forward_strided_dropout", "na1d_fused_backward_strided_dropout",
                       "na1d_version", "na1d_status_string")
 UNSUPPORTED = -8
 
@@ -73,6 +74,12 @@ def load():
     lib.na1d_global_backward.argtypes = [_ptr] * 10 + [_i64] * 4 + [_f32, _int, _f32, _u64, _ptr, _i64, _ptr]
     lib.na1d_global_backward_workspace_bytes.restype = _i64
     lib.na1d_global_backward_workspace_bytes.argtypes = [_i64] * 4 + [_int]
+    lib.na1d_fused_forward_strided_dropout.restype = _int
+    lib.na1d_fused_forward_strided_dropout.argtypes = [_ptr] * 7 + [_i64] * 6 + [_f32, _int, _ptr, _ptr, _f32, _u64,
+                                                                              _i64, _i64, _i64, _ptr]
+    lib.na1d_fused_backward_strided_dropout.restype = _int
+    lib.na1d_fused_backward_strided_dropout.argtypes = [_ptr] * 11 + [_i64] * 6 + [_f32, _int, _ptr, _ptr, _f32, _u64,
+                                                                                _i64, _i64, _i64, _ptr, _i64, _ptr]
     lib.na1d_fused_backward_noalloc.restype = _int
     lib.na1d_fused_backward_noalloc.argtypes = [_ptr] * 12 + [_i64] * 6 + [_f32, _int, _ptr]
     lib.na1d_force_generic.restype = _int
@@ -165,29 +172,44 @@ def _strides3(view):
     return (_i64 * 3)(view.stride(0), view.stride(1), view.stride(2))
 
 
-def call_fused_forward_strided(out, lse, q, k, v, rpb, t_valid, W, left, scale):
+def call_fused_forward_strided(out, lse, q, k, v, rpb, t_valid, W, left, scale, dropout=None):
     """q, k, v, out: ``[N, H, T, C]`` views (q, k, v with equal strides).  Returns the status so that the
-    caller can pack the tensors when no strided kernel covers the shape (``UNSUPPORTED``)."""
+    caller can pack the tensors when no strided kernel covers the shape (``UNSUPPORTED``).  ``dropout``: ``None`` or
+    ``(p, seed, row_stride, row_offset, seq_rows)`` - see na1d_fused_forward_strided_dropout."""
     lib = load()
     N, H, T, C = q.shape
     assert q.stride() == k.stride() == v.stride()
     with torch.cuda.device(out.device):
-        st = lib.na1d_fused_forward_strided(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid), N, H, T, C, W,
-                                            left, scale, dtype_tag(q.dtype), _strides3(q), _strides3(out), _stream(out))
+        if dropout is None:
+            st = lib.na1d_fused_forward_strided(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid), N, H, T, C,
+                                                W, left, scale, dtype_tag(q.dtype), _strides3(q), _strides3(out),
+                                                _stream(out))
+        else:
+            st = lib.na1d_fused_forward_strided_dropout(_p(out), _p(lse), _p(q), _p(k), _p(v), _p(rpb), _p(t_valid), N,
+                                                        H, T, C, W, left, scale, dtype_tag(q.dtype), _strides3(q),
+                                                        _strides3(out), *dropout, _stream(out))
     if st != UNSUPPORTED:
         check(st, "na1d_fused_forward_strided")
     return st
 
 
-def call_fused_backward_strided(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, W, left, scale, workspace=None):
+def call_fused_backward_strided(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, W, left, scale, workspace=None,
+                                dropout=None):
     lib = load()
     N, H, T, C = q.shape
     assert q.stride() == k.stride() == v.stride() == dq.stride() == dk.stride() == dv.stride()
     ws_bytes = 0 if workspace is None else workspace.numel() * workspace.element_size()
     with torch.cuda.device(dq.device):
-        st = lib.na1d_fused_backward_strided(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(dout), _p(lse),
-                                             _p(rpb), _p(t_valid), N, H, T, C, W, left, scale, dtype_tag(q.dtype),
-                                             _strides3(q), _strides3(dout), _p(workspace), ws_bytes, _stream(dq))
+        if dropout is None:
+            st = lib.na1d_fused_backward_strided(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v), _p(dout),
+                                                 _p(lse), _p(rpb), _p(t_valid), N, H, T, C, W, left, scale,
+                                                 dtype_tag(q.dtype), _strides3(q), _strides3(dout), _p(workspace),
+                                                 ws_bytes, _stream(dq))
+        else:
+            st = lib.na1d_fused_backward_strided_dropout(_p(dq), _p(dk), _p(dv), _p(drpb), _p(q), _p(k), _p(v),
+                                                         _p(dout), _p(lse), _p(rpb), _p(t_valid), N, H, T, C, W, left,
+                                                         scale, dtype_tag(q.dtype), _strides3(q), _strides3(dout),
+                                                         *dropout, _p(workspace), ws_bytes, _stream(dq))
     if st != UNSUPPORTED:
         check(st, "na1d_fused_backward_strided")
     return st

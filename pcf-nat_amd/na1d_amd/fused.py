@@ -22,11 +22,14 @@ def _residue_lengths(t_valid, r, d):
     return None if t_valid is None else ((t_valid - r + d - 1) // d).clamp_(min=0).to(torch.int32)
 
 
-def _strided_or_packed_forward(out4, lse, q4, k4, v4, rpb, t_valid, W, left, scale):
+def _strided_or_packed_forward(out4, lse, q4, k4, v4, rpb, t_valid, W, left, scale, dropout=None):
     """Forward on ``[N, H, T, C]`` views through the strided entry point, or - for shapes it does not cover -
-    on packed copies through the packed one.  Returns the packed output when it had to be made."""
-    if _lib.call_fused_forward_strided(out4, lse, q4, k4, v4, rpb, t_valid, W, left, scale) == 0:
+    on packed copies through the packed one.  Returns the packed output when it had to be made.  ``dropout``:
+    ``None`` or ``(p, seed, row_stride, row_offset, seq_rows)``."""
+    if _lib.call_fused_forward_strided(out4, lse, q4, k4, v4, rpb, t_valid, W, left, scale, dropout=dropout) == 0:
         return None
+    if dropout is not None:
+        raise _lib.NA1DError("attention dropout needs head_dim <= 128 (no dropout on the generic kernels)")
     N, H, T, C = q4.shape
     qp, kp, vp = (z.contiguous().view(N * H, T, C) for z in (q4, k4, v4))
     op = torch.empty_like(qp)
@@ -35,10 +38,11 @@ def _strided_or_packed_forward(out4, lse, q4, k4, v4, rpb, t_valid, W, left, sca
     return op
 
 
-def _strided_or_packed_backward(dq4, dk4, dv4, drpb, q4, k4, v4, packed_out, dout4, lse, rpb, t_valid, W, left, scale, ws):
+def _strided_or_packed_backward(dq4, dk4, dv4, drpb, q4, k4, v4, packed_out, dout4, lse, rpb, t_valid, W, left, scale, ws,
+                                dropout=None):
     if packed_out is None:
         st = _lib.call_fused_backward_strided(dq4, dk4, dv4, drpb, q4, k4, v4, dout4, lse, rpb, t_valid, W, left, scale,
-                                              workspace=ws)
+                                              workspace=ws, dropout=dropout)
         assert st == 0
         return
     N, H, T, C = q4.shape
@@ -66,7 +70,6 @@ class _FusedNA1D(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, rpb, t_valid, num_heads, win_size, left, scale, deterministic, dilation, dropout):
         assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
-        assert dropout is None or dilation == 1, "attention dropout is defined for dilation 1"
         ctx.dropout = dropout
         assert q.dtype == k.dtype == v.dtype
         assert q.dim() == 3 and q.shape == k.shape == v.shape, "q, k, v must all be [B, T, C]"
@@ -96,7 +99,8 @@ class _FusedNA1D(torch.autograd.Function):
             lse = torch.empty((B, qr.shape[2]), dtype=torch.float32, device=q.device)
             ctx.packed_outs.append(_strided_or_packed_forward(
                 _residue(o4, r, dilation), lse, qr, _residue(k4, r, dilation), _residue(v4, r, dilation), rpb,
-                _residue_lengths(t_valid, r, dilation), win_size, left, scale))
+                _residue_lengths(t_valid, r, dilation), win_size, left, scale,
+                dropout=None if dropout is None else (*dropout, dilation, r, T)))     # rows named by their place in T
             lses.append(lse)
         ctx.save_for_backward(q, k, v, out, rpb, t_valid, *lses)
         return out
@@ -122,7 +126,8 @@ class _FusedNA1D(torch.autograd.Function):
             for r, lse in enumerate(lses):
                 a = [_residue(z, r, dilation) for z in views]
                 _strided_or_packed_backward(a[0], a[1], a[2], drpb, a[3], a[4], a[5], ctx.packed_outs[r], a[6], lse, rpb,
-                                            _residue_lengths(t_valid, r, dilation), win_size, left, scale, ws)
+                                            _residue_lengths(t_valid, r, dilation), win_size, left, scale, ws,
+                                            dropout=None if ctx.dropout is None else (*ctx.dropout, dilation, r, T))
         if drpb is not None:
             drpb = drpb.view(ctx.rpb_shape)
         return dq, dk, dv, drpb, None, None, None, None, None, None, None, None
@@ -146,7 +151,9 @@ def na1d_fused(q, k, v, win_size, left, rpb=None, t_valid=None, num_heads=1, sca
     dropout_p, seed : attention dropout inside the kernels (nn.Dropout(attn_drop) of models/PCF_NATransformer.py:71,149):
               each probability is kept with chance ``1 - dropout_p`` and scaled by ``1 / (1 - dropout_p)``.  The mask
               is a hash of (seed, sequence, row, window slot) that the backward recomputes; ``seed`` (a 64-bit int)
-              defaults to a draw from torch's CPU generator.  Needs ``dilation == 1`` and head_dim <= 128.
+              defaults to a draw from torch's CPU generator.  Needs head_dim <= 128.  With ``dilation > 1`` the mask
+              is still the one of (sequence, row, slot) of the whole operator: the launches on the residue classes
+              name their rows by their place in the sequence.
     Returns ``[B, T, C]`` in q's dtype.  The gradient of ``rpb`` has rpb's shape.
     """
     dropout = None

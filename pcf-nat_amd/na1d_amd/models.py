@@ -394,7 +394,6 @@ class NAttention(nn.Module):
         nn.init.normal_(self.relative_position_bias, mean=0.0, std=0.02)
         self.proj = _Projection.make(dim, dim, True, groups, channels_first)
         self.register_buffer("attn_mask", _window_mask(frames, win_size, left, None, torch.float32, "cpu").unsqueeze(1))
-        assert attn_drop == 0.0 or dilation == 1, "attention dropout is built for dilation 1"
         if na == "unfused":     # like the reference's CUDA path, the two-call chain has no dilated kernels
             self.NA1d_QK_Function, self.NA1d_AV_Function = getNA1dFunction(C=head_dim, dilation=dilation, dtype=dtype)
 

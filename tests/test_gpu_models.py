@@ -161,6 +161,24 @@ def test_attention_dropout_in_training_only(na):
     assert g is not None and torch.isfinite(g).all() and g.abs().sum() > 0
 
 
+def test_dilated_layer_drops_in_training_only():
+    """A dilated layer (the reference runs these on the CPU only, models/PCF_NATransformer.py:158-170) with
+    attn_drop: eval is the plain layer, training draws a fresh mask per call and has finite gradients."""
+    torch.manual_seed(3)
+    layer = models.NAttention(frames=90, dim=64, num_heads=4, win_size=15, groups=1, channels_first=True, na="fused",
+                              dilation=3, attn_drop=0.25).cuda().to(torch.bfloat16)
+    plain = models.NAttention(frames=90, dim=64, num_heads=4, win_size=15, groups=1, channels_first=True, na="fused",
+                              dilation=3).cuda().to(torch.bfloat16)
+    plain.load_state_dict(layer.state_dict())
+    x = torch.randn(3, 64, 90, generator=torch.Generator().manual_seed(4)).cuda().to(torch.bfloat16).requires_grad_(True)
+    with torch.no_grad():
+        assert torch.equal(layer.eval()(x), plain.eval()(x))
+    a, b = layer.train()(x), layer(x)
+    assert torch.isfinite(a).all() and not torch.equal(a, b)
+    a.float().sum().backward()
+    assert torch.isfinite(x.grad).all() and x.grad.abs().sum() > 0
+
+
 @pytest.mark.parametrize("na", ["fused", "fused_qkv"])
 def test_mfa_nat_4x4_inference_with_lengths_fp16(na):
     """The tokens-first family in inference (fused_qkv: the token-major pipeline with folded batch norms, the

@@ -629,6 +629,64 @@ def test_dropout_mask_is_bit_exact(W, L):
     assert ((kept * (1 - p) * W).round() >= 1).all()                 # survivors carry 1 / (1 - p)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+@pytest.mark.parametrize("geom,dilation", [((2, 2, 61, 32, 15, 7), 2), ((2, 4, 100, 16, 27, 13), 3), ((1, 2, 150, 64, 33, 16), 2),
+                                           ((2, 2, 47, 24, 9, 0), 4), ((2, 1, 90, 32, 65, 32), 2), ((2, 2, 5, 16, 27, 13), 7)],
+                         ids=lambda g: "x".join(map(str, g)) if isinstance(g, tuple) else "d%d" % g)
+def test_fused_dropout_with_dilated_windows_matches_oracle(geom, dilation, dtype):
+    """The launches on the residue classes drop by (sequence, row, slot) of the whole operator: same oracle mask as
+    for dilation 1, applied to the dilated window (models/PCF_NATransformer.py:149 with :158-170)."""
+    N, H, T, C, W, L = geom
+    B, p, seed = N * H, 0.3, 0x0FED_CBA9_8765_4321
+    q, k, v, do = make_inputs(B, T, C, W, 52, dtype, n=4, scale=C ** -0.5)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(7)) * 0.5
+    pad = torch.tensor([0, T // 3][:N])
+    t_valid = (T - pad).to(torch.int32).cuda()
+    print("fused dropout dilated", geom, dilation, dtype, flush=True)
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    rd = rpb.cuda().requires_grad_(True)
+    out = na1d_fused(qd, kd, vd, W, L, rpb=rd, t_valid=t_valid, num_heads=H, dilation=dilation, dropout_p=p, seed=seed)
+    out.backward(do.cuda())
+    keep = O.dropout_keep(B, T, W, p, seed)
+    qf, kf, vf = q.float(), k.float(), v.float()
+    want_o, _, _ = O.na1d_forward(qf, kf, vf, W, L, rpb, pad, H, dilation, keep=keep, p_drop=p)
+    wq, wk, wv, wr = O.na1d_backward(qf, kf, vf, do.float(), W, L, rpb, pad, H, dilation, keep=keep, p_drop=p)
+    tol = TOL[dtype]
+    assert O.rel_l2(out.float(), want_o) < tol, "O"
+    assert O.rel_l2(qd.grad.float(), wq) < tol, "dQ"
+    assert O.rel_l2(kd.grad.float(), wk) < tol, "dK"
+    assert O.rel_l2(vd.grad.float(), wv) < tol, "dV"
+    assert _err(rd.grad, wr) < tol, "drpb"
+
+
+@pytest.mark.parametrize("W,L,dilation", [(15, 7, 2), (27, 13, 3), (65, 32, 2), (9, 0, 5)])
+def test_dilated_dropout_mask_is_bit_exact(W, L, dilation):
+    """As test_dropout_mask_is_bit_exact, with slot j of row t at column t + (j - L) * dilation."""
+    B, T, C, p, seed = 3, 100, 128, 0.5, 77
+    q = torch.zeros(B, T, C, dtype=torch.float16, device="cuda")
+    v = torch.zeros(B, T, C, dtype=torch.float16)
+    v[:, torch.arange(T), torch.arange(T)] = 1.0
+    out = na1d_fused(q, q, v.cuda(), W, L, dilation=dilation, dropout_p=p, seed=seed).cpu()
+    keep = O.dropout_keep(B, T, W, p, seed)
+    want = torch.zeros(B, T, C, dtype=torch.bool)
+    for j in range(W):
+        off = (j - L) * dilation
+        rows = torch.arange(max(0, -off), min(T, T - off))
+        if rows.numel():
+            want[:, rows, rows + off] = keep[:, rows, j]
+    assert torch.equal(out != 0, want)
+
+
+def test_strided_dropout_rejects_rows_outside_the_sequence():
+    q = torch.zeros(2, 2, 20, 32, dtype=torch.bfloat16, device="cuda")
+    lse = torch.empty(4, 20, device="cuda")
+    ok = _lib.call_fused_forward_strided(torch.empty_like(q), lse, q, q, q, None, None, 5, 2, 1.0, dropout=(0.5, 1, 2, 1, 40))
+    assert ok == 0
+    for bad in [(0.5, 1, 2, 2, 40), (0.5, 1, 2, 1, 39), (0.5, 1, 0, 0, 40), (1.0, 1, 1, 0, 20)]:
+        with pytest.raises(_lib.NA1DError):
+            _lib.call_fused_forward_strided(torch.empty_like(q), lse, q, q, q, None, None, 5, 2, 1.0, dropout=bad)
+
+
 def test_dropout_rate_zero_is_the_plain_operator_and_bad_rates_are_rejected():
     q, k, v = dev(*make_inputs(4, 50, 32, 15, 3, torch.bfloat16))
     assert torch.equal(na1d_fused(q, k, v, 15, 7, dropout_p=0.0), na1d_fused(q, k, v, 15, 7))
