@@ -313,6 +313,12 @@ drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, 
     if (threadIdx.x == 0) drpb[h * W + j] += acc[0];
 }
 
+// Waves per SIMD the register allocation of the backward must leave room for.  16-channel heads: the LDS footprint
+// admits six workgroups per CU, so the registers must too (80 or fewer; the dropout variant would spill and is left alone).
+#ifndef NA1D_BWD_MIN_WAVES
+#define NA1D_BWD_MIN_WAVES(C, DROP) ((C) == 16 && !(DROP) ? 6 : 1)
+#endif
+
 template <int C> struct StripBwd {
 #ifdef NA1D_BWD_MT
     static constexpr int kMaxTiles = NA1D_BWD_MT * 32 / (C < 32 ? 32 : C);
@@ -322,7 +328,7 @@ template <int C> struct StripBwd {
 };
 
 template <class DT, int C, int NBV, bool DROP>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kThreads, NA1D_BWD_MIN_WAVES(C, DROP))
 fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, float *__restrict__ drpb,
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
@@ -349,7 +355,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     const int key_region = region_bytes<C>(nt + 1 + NBV), qry_region = region_bytes<C>(nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
-    LDS_PTR(char) sc_lds = k_lds;                  // score tiles [(tq*2 + X/Y)*2 + P/dS]
+    LDS_PTR(char) sc_lds = k_lds;                  // score tiles [((tq - sc_skip)*2 + X/Y)*2 + P/dS]
     LDS_PTR(char) q_lds = k_lds + kv_bytes;
     LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
     LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
@@ -361,6 +367,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     const uint32_t item = wi.item, b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
     const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
+    const int sc_skip = strips == 1 ? 1 : 0;       // a strip that is the whole sequence has no halo tiles to keep scores of
 
     const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
     {
@@ -552,8 +559,9 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 #pragma unroll
     for (int jt = 0; jt < TPW; ++jt) {
         const int tq = wave + jt * kWaves;
-        if (tq > nt + 1) continue;
-        LDS_PTR(char) t = sc_lds + tq * 4 * kScoreTile + n * 32 + g * 8;     // tile[query n][key slots 4g..4g+3]
+        const int qt = i0 - 1 + tq;
+        if (qt > i1 || qt < 0 || qt >= tiles) continue;                      // no such tile: pass 2 does not look for it
+        LDS_PTR(char) t = sc_lds + (tq - sc_skip) * 4 * kScoreTile + n * 32 + g * 8;   // tile[query n][key slots 4g..4g+3]
 #pragma unroll
         for (int xy = 0; xy < 2; ++xy)
 #pragma unroll
@@ -586,18 +594,24 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         for (int ct = 0; ct < CT; ++ct) acck[ct] = accv[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
+            // a query tile outside the sequence (its Q and dO rows were staged as zeros) has no score tile: read one
+            // that is there and drop what it holds
+            const bool there = (uint32_t)(kp - vb) < (uint32_t)tiles;
+            const uint32_t tm = there ? 0xffffffffu : 0u;
             const int tq = kp - vb - (i0 - 1);
             LDS_PTR(char) qtile = q_lds + tq * LL::kTileBytes;
             LDS_PTR(char) gtile = g_lds + tq * LL::kTileBytes;
-            LDS_PTR(char) stile = sc_lds + (tq * 4 + (vb == 1 ? 2 : 0)) * kScoreTile + sc_lane;
+            LDS_PTR(char) stile = sc_lds + (((there ? tq : 1) - sc_skip) * 4 + (vb == 1 ? 2 : 0)) * kScoreTile + sc_lane;
             u32x2 pb = read_tr(stile), db = read_tr(stile + kScoreTile);
             if (NBV == 3 && vb == 0) {
-                pb = u32x2{pb.x & keep0t.x, pb.y & keep0t.y};
-                db = u32x2{db.x & keep0t.x, db.y & keep0t.y};
-            }
-            if (NBV == 3 && vb == 2) {
-                pb = u32x2{pb.x & ~keep0t.x, pb.y & ~keep0t.y};
-                db = u32x2{db.x & ~keep0t.x, db.y & ~keep0t.y};
+                pb = u32x2{pb.x & keep0t.x & tm, pb.y & keep0t.y & tm};
+                db = u32x2{db.x & keep0t.x & tm, db.y & keep0t.y & tm};
+            } else if (NBV == 3 && vb == 2) {
+                pb = u32x2{pb.x & ~keep0t.x & tm, pb.y & ~keep0t.y & tm};
+                db = u32x2{db.x & ~keep0t.x & tm, db.y & ~keep0t.y & tm};
+            } else {
+                pb = u32x2{pb.x & tm, pb.y & tm};
+                db = u32x2{db.x & tm, db.y & tm};
             }
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
@@ -640,7 +654,8 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     auto kern = g.drop.threshold ? (two ? fused_bwd_kernel<DT, C, 2, true> : fused_bwd_kernel<DT, C, 3, true>)
                                  : (two ? fused_bwd_kernel<DT, C, 2, false> : fused_bwd_kernel<DT, C, 3, false>);
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
-    const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + 2) * 4 * 512);
+    // (a strip that is the whole sequence has no halo tiles)
+    const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + (sp.strips == 1 ? 0 : 2)) * 4 * 512);
     const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
                        (kThreads + kBiasEntries + (drpb ? kWaves * 32 : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
