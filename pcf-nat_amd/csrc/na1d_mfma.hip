@@ -14,13 +14,18 @@ namespace mfma {
 #define NA1D_HG_MT 4
 #endif
 constexpr int kGroupTiles = NA1D_HG_MT;      // tiles per strip when heads are staged in groups
+#ifndef NA1D_HG_WAVES
+#define NA1D_HG_WAVES 8
+#endif
+constexpr int kGroupWaves = NA1D_HG_WAVES;   // waves per workgroup when heads are staged in groups: a group's regions are
+                                             // 2-4 times a head's, and twice the waves keep as many tiles in flight per CU
 
 // HG heads whose rows lie side by side in memory (a projection's output, head h of a token right behind head h-1)
 // can be staged together: the strip copies then move HG * C channels of a row in one piece - whole 128-byte lines
 // for four heads of 16 channels, where a head alone would ask for quarter lines - into regions laid out as rows of
-// C * HG channels, and every wave computes the tiles of one head (kWaves / HG waves share a head's tiles).
+// C * HG channels, and every wave computes the tiles of one head (kGroupWaves / HG waves share a head's tiles).
 template <class DT, int C, int NBV, bool DROP, int HG>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(64 * (HG > 1 ? kGroupWaves : kWaves))
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
@@ -28,10 +33,11 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
                  int shift_arg, Dropout drop) {
     const int shift = NBV == 3 ? 16 : shift_arg;     // three key blocks always start one tile before the query tile
     constexpr int CS = C * HG;                       // channels of a staged row
+    constexpr int NW = HG > 1 ? kGroupWaves : kWaves; // waves of the workgroup
     using LL = Lds<CS>;
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = HG > 1 ? kGroupTiles : Strip<CS>::kMaxTiles;
-    static_assert(kWaves % HG == 0, "whole waves per head");
+    static_assert(NW % HG == 0, "whole waves per head");
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
@@ -68,16 +74,16 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         const int lane_off = direct_lane_offset<CS>(wave, lane, in.pitch, HG * in.width);
         const bool whole_lines = in.pitch == 2 * C || CS % 64 == 0;
         if (strips == 1 && whole_lines) {      // nobody else reads these rows' lines
-            stage_direct<CS, MT + 2, kReadOnce>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
-            stage_direct<CS, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-            stage_direct<CS, MT + 2, kReadOnce>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, kReadOnce, NW>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<CS, MT, kReadOnce, NW>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, kReadOnce, NW>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
         } else {
-            stage_direct<CS, MT + 2, kReadShared>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, kReadShared, NW>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
             if (whole_lines)
-                stage_direct<CS, MT, kReadOnce>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+                stage_direct<CS, MT, kReadOnce, NW>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
             else
-                stage_direct<CS, MT, kReadShared>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-            stage_direct<CS, MT + 2, kReadShared>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+                stage_direct<CS, MT, kReadShared, NW>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, kReadShared, NW>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
         }
     }
 
@@ -104,7 +110,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     read_window<NBV>(win, bias_lds, L, shift, g, n);
     __syncthreads();
 
-    for (int i = i0 + wave / HG; i < i1; i += kWaves / HG) {
+    for (int i = i0 + wave / HG; i < i1; i += NW / HG) {
         const int tile_bytes = (i - i0) * LL::kTileBytes;
         RowOperand<C> qt;
         read_rows<C>(qt, q_lds + tile_bytes, q_lane);
@@ -213,14 +219,14 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         // region, leave as whole lines - the strip copy run backwards, each lane taking the 16-byte unit that sits
         // at its place in LDS to where it belongs in memory.
         __syncthreads();
-        constexpr int kRounds = (region_bytes<CS>(MT) / kChunk + kWaves - 1) / kWaves;
+        constexpr int kRounds = (region_bytes<CS>(MT) / kChunk + NW - 1) / NW;
         constexpr int kChunkRows = kChunk / LL::kRowBytes;
         const Rsrc gs = make_rsrc(out + sample * outl.sample + head0 * outl.head, min(T, 16 * i1) * outl.pitch);
         const int lane_off = direct_lane_offset<CS>(wave, lane, outl.pitch, HG * outl.width);
         const int chunks = region_bytes<CS>(i1 - i0) / kChunk;
 #pragma unroll
         for (int j = 0; j < kRounds; ++j) {
-            const int c = j * kWaves + wave;
+            const int c = j * NW + wave;
             if (c < chunks) {
                 const u32x4 unit = *reinterpret_cast<LDS_PTR(u32x4)>(q_lds + c * kChunk + lane * 16);
                 __builtin_amdgcn_raw_buffer_store_b128(unit, gs, (16 * i0 + c * kChunkRows) * outl.pitch + lane_off, 0, kStoreAux);
@@ -251,7 +257,8 @@ int launch_fwd_hg(void *out, float *lse, const void *q, const void *k, const voi
                        HG * kBiasEntries * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     note_kernel("fused_fwd_kernel", DT::tag, C, two ? 2 : 3, g.drop.threshold != 0, HG);
-    launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
+    launch_kernel_block(kern, (unsigned)sp.items, 64u * (HG > 1 ? kGroupWaves : kWaves), lds, s, (char *)out, lse,
+                  (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
                   div_magic(sp.strips), div_magic(g.H / HG), byte_strides(in, g), byte_strides(outl, g), window_shift(g),
                   g.drop);

@@ -167,16 +167,17 @@ __device__ inline int direct_lane_offset(int wave, int lane, int pitch = Lds<C>:
     const int unit = su ^ Lds<C>::swz(u / Lds<C>::kUnits);
     return unit * 16 < width ? (lane / Lds<C>::kUnits) * pitch + unit * 16 : kNowhere;
 }
-template <int C, int NTILES, int AUX>
+template <int C, int NTILES, int AUX, int NW = kWaves>       // NW: the waves of the workgroup that share the copy
 __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, int ntiles, int wave, int lane_off,
                                     int pitch = Lds<C>::kRowBytes) {
-    constexpr int kRounds = (region_bytes<C>(NTILES) / kChunk + kWaves - 1) / kWaves;
+    static_assert(NW % 4 == 0, "chunk -> swizzle phase mapping assumes a multiple of four waves");
+    constexpr int kRounds = (region_bytes<C>(NTILES) / kChunk + NW - 1) / NW;
     constexpr int kChunkRows = kChunk / Lds<C>::kRowBytes;
     const int chunks = region_bytes<C>(ntiles) / kChunk;
     const int base = row_lo * pitch + lane_off, step = kChunkRows * pitch;
 #pragma unroll
     for (int j = 0; j < kRounds; ++j) {
-        const int c = j * kWaves + wave;
+        const int c = j * NW + wave;
         if (c < chunks)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * kChunk), 16, base + c * step, 0, 0, AUX);
     }
