@@ -123,6 +123,31 @@ def test_dropout_entry_points_validate():
     assert b(*bargs(lse=None)) == -1 and b(*bargs(p=1.5)) == -5
 
 
+def test_strided_dropout_entry_points_validate():
+    lib = _lib.load()
+    ok = ctypes.c_void_p(0x1000)
+    S = lambda *v: (ctypes.c_int64 * 3)(*v)
+    qkv, out = S(8 * 3 * 2 * 16, 16, 3 * 2 * 16), S(8 * 2 * 16, 16, 2 * 16)     # [N, T, 3, H, C] / [N, T, H*C], T=8, H=2, C=16
+    f = lib.na1d_fused_forward_strided_dropout
+    args = lambda **kw: [ok, None, ok, ok, kw.get("v", ok), None, None, kw.get("N", 2), 2, 8, kw.get("C", 16), 5, 2, 1.0, 0,
+                         kw.get("qs", qkv), out, kw.get("p", 0.5), 7, kw.get("stride", 2), kw.get("offset", 1),
+                         kw.get("rows", 16), None]
+    assert f(*args(v=None)) == -1 and f(*args(qs=None)) == -1 and f(*args(C=20)) == -3
+    assert f(*args(p=1.0)) == -5 and f(*args(p=float("nan"))) == -5
+    assert f(*args(stride=0)) == -5 and f(*args(offset=2)) == -5 and f(*args(offset=-1)) == -5
+    assert f(*args(rows=15)) == -5                   # row 1 + 2 * 7 = 15 needs 16 rows
+    assert f(*args(rows=1 << 31)) == -5
+    assert f(*args(N=0)) == 0                        # nothing to do
+    assert f(*args(C=136, qs=S(8 * 3 * 2 * 136, 136, 3 * 2 * 136))) in (-5, -8)
+    b = lib.na1d_fused_backward_strided_dropout
+    bargs = lambda **kw: [ok, ok, ok, None, ok, ok, ok, kw.get("g", ok), kw.get("lse", ok), None, None, 2, 2, 8, 16, 5, 2,
+                          1.0, 0, qkv, out, kw.get("p", 0.5), 7, kw.get("stride", 2), 1, kw.get("rows", 16),
+                          kw.get("ws", None), 64, None]
+    assert b(*bargs(lse=None)) == -1 and b(*bargs(g=None)) == -1 and b(*bargs(p=1.5)) == -5
+    assert b(*bargs(stride=0)) == -5 and b(*bargs(rows=15)) == -5
+    assert b(*bargs(ws=ctypes.c_void_p(0x1008))) == -6
+
+
 def test_dense_attention_entry_points_validate():
     lib = _lib.load()
     P, ok = ctypes.c_void_p, ctypes.c_void_p(0x1000)
