@@ -36,7 +36,7 @@ constexpr int kBandMaxTiles = 8;          // compile-time ceiling of max_tiles
 // rows the strip needs.  `first` is a tile start, so 16-byte units never straddle the sequence's start.
 // The region is padded to whole chunks (score_bytes).
 inline __host__ __device__ int score_bytes(int tiles, int W) { return (tiles * 16 * W * 4 + kChunk - 1) / kChunk * kChunk; }
-template <int NBV>
+template <int NBV, int AUX>
 __device__ inline void stage_scores(Rsrc src, int first, LDS_PTR(float) region, int tiles, int W, int wave, int lane) {
     // at most kBandMaxTiles + NBV tiles of 16 rows of W <= 16*NBV - 15 floats
     constexpr int kRounds = (((kBandMaxTiles + NBV) * 16 * (16 * NBV - 15) * 4 + kChunk - 1) / kChunk + kWaves - 1) / kWaves;
@@ -46,7 +46,7 @@ __device__ inline void stage_scores(Rsrc src, int first, LDS_PTR(float) region, 
         const int c = j * kWaves + wave;
         if (c < chunks)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * (kChunk / 4)), 16,
-                                                     first * 4 + c * kChunk + lane * 16, 0, 0, kReadShared);
+                                                     first * 4 + c * kChunk + lane * 16, 0, 0, AUX);
     }
 }
 
@@ -85,8 +85,13 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     {
         const int key_bytes = min(T, 16 * (i0 - sb + kt)) * pitch, qry_bytes = min(T, 16 * i1) * pitch;
         const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
-        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off, pitch);
-        stage_direct<C, MT, kReadShared>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off, pitch);
+        if (strips == 1) {      // nobody else reads these rows
+            stage_direct<C, MT + NBV, kReadOnce>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off, pitch);
+            stage_direct<C, MT, kReadOnce>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off, pitch);
+        } else {                // (the read-once policy on the query rows alone measured 8 % slower at T = 300)
+            stage_direct<C, MT + NBV, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off, pitch);
+            stage_direct<C, MT, kReadShared>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off, pitch);
+        }
     }
     const Rsrc as = make_rsrc(attn + (int64_t)b * T * W, T * W * 4);
     RowLane<C> k_lane, q_lane;
@@ -156,9 +161,13 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
     const int64_t seq_off = (int64_t)b * T * pitch;      // packed rows of head_dim = pitch / 2 channels
     {
         const int key_bytes = min(T, 16 * (i0 - sb + kt)) * pitch;
-        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(v + seq_off, key_bytes), 16 * (i0 - sb), v_lds, kt, wave,
-                                               direct_lane_offset<C>(wave, lane, pitch, pitch), pitch);
-        stage_scores<NBV>(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, s_lds, nt, W, wave, lane);
+        const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
+        if (strips == 1)        // nobody else reads these rows
+            stage_direct<C, MT + NBV, kReadOnce>(make_rsrc(v + seq_off, key_bytes), 16 * (i0 - sb), v_lds, kt, wave, lane_off, pitch);
+        else
+            stage_direct<C, MT + NBV, kReadShared>(make_rsrc(v + seq_off, key_bytes), 16 * (i0 - sb), v_lds, kt, wave, lane_off, pitch);
+        // the strip's own score rows: read once (at most the line at either end is shared with a neighbour)
+        stage_scores<NBV, kReadOnce>(make_rsrc(attn + (int64_t)b * T * W, min(T, 16 * i1) * W * 4), 16 * i0 * W, s_lds, nt, W, wave, lane);
     }
     const Rsrc os = make_rsrc(out + seq_off, T * pitch);
     TrLane<C> v_lane;
@@ -221,9 +230,14 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     const int64_t seq_off = (int64_t)b * T * pitch;      // packed rows of head_dim = pitch / 2 channels
     {
         const int rows_hi = min(T, 16 * (q0 + qtiles));
-        stage_direct<C, MT + NBV, kReadShared>(make_rsrc(x + seq_off, rows_hi * pitch), 16 * q0, x_lds, qtiles, wave,
-                                               direct_lane_offset<C>(wave, lane, pitch, pitch), pitch);
-        stage_scores<NBV>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), 16 * q0 * W, s_lds, qtiles, W, wave, lane);
+        const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
+        if (strips == 1) {      // nobody else reads these rows
+            stage_direct<C, MT + NBV, kReadOnce>(make_rsrc(x + seq_off, rows_hi * pitch), 16 * q0, x_lds, qtiles, wave, lane_off, pitch);
+            stage_scores<NBV, kReadOnce>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), 16 * q0 * W, s_lds, qtiles, W, wave, lane);
+        } else {
+            stage_direct<C, MT + NBV, kReadShared>(make_rsrc(x + seq_off, rows_hi * pitch), 16 * q0, x_lds, qtiles, wave, lane_off, pitch);
+            stage_scores<NBV, kReadShared>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), 16 * q0 * W, s_lds, qtiles, W, wave, lane);
+        }
     }
     TrLane<C> x_tr;
     x_tr.init(0, lane);
