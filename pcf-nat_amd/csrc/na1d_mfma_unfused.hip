@@ -65,8 +65,8 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     using LL = Lds<C>;
     constexpr int MT = kBandMaxTiles;
     fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
-    // dynamic LDS: K region of kt tiles starting sb tiles before the strip, Q region of nt tiles, one 16 x W fp32
-    // tile per wave
+    // dynamic LDS: K region of kt tiles starting sb tiles before the strip, Q region of nt tiles, two 16 x W fp32
+    // tiles per wave
     const int sb = (shift + 15) >> 4, kt = nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
@@ -97,23 +97,30 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     RowLane<C> k_lane, q_lane;
     k_lane.init(16 * sb - shift, lane);
     q_lane.init(0, lane);
-    LDS_PTR(float) mine = out_lds + wave * 16 * W;
+    LDS_PTR(float) mine = out_lds + wave * 32 * W;
     wait_direct();
     __syncthreads();
 
-    for (int i = i0 + wave; i < i1; i += kWaves) {
-        const int tile_bytes = (i - i0) * LL::kTileBytes;
-        RowOperand<C> qt;
-        read_rows<C>(qt, q_lds + tile_bytes, q_lane);
+    // A wave takes two neighbouring tiles at a time: their 32*W floats are a run of W whole 128-byte lines (where the
+    // sequence's rows start on a line), which leaves as one streaming write instead of two pieces per tile that L2
+    // has to merge.
+    for (int i = i0 + 2 * wave; i < i1; i += 2 * kWaves) {
+        const int pair = min(2, i1 - i);
+        for (int h = 0; h < pair; ++h) {
+            const int tile_bytes = (i + h - i0) * LL::kTileBytes;
+            LDS_PTR(float) tile = mine + h * 16 * W;
+            RowOperand<C> qt;
+            read_rows<C>(qt, q_lds + tile_bytes, q_lane);
 #pragma unroll
-        for (int vb = 0; vb < NBV; ++vb) {
-            RowOperand<C> kop;
-            read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
-            const f32x4 s = dot_rows_mma<DT, C>(kop, qt);
+            for (int vb = 0; vb < NBV; ++vb) {
+                RowOperand<C> kop;
+                read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
+                const f32x4 s = dot_rows_mma<DT, C>(kop, qt);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int j = 16 * vb + 4 * g + r - shift - n + L;
-                if (j >= 0 && j < W) mine[n * W + j] = s[r];      // every (row, slot) is written by exactly one lane
+                for (int r = 0; r < 4; ++r) {
+                    const int j = 16 * vb + 4 * g + r - shift - n + L;
+                    if (j >= 0 && j < W) tile[n * W + j] = s[r];  // every (row, slot) is written by exactly one lane
+                }
             }
         }
         // LDS serves one wave's accesses in program order, so the other lanes' values are there when the
@@ -121,14 +128,9 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
         const int first = 16 * i * W;                             // floats into the sequence's score rows
-        if (W % 2 == 0) {       // a tile's 16*W floats are whole 128-byte lines: written once, by this wave alone
-            for (int u = lane; u * 4 < 16 * W; u += 64)
-                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, kStoreAux);
-        } else {                // neighbouring tiles share the first and last line: let L2 merge them
-            for (int u = lane; u * 4 < 16 * W; u += 64)
-                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, 0);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");    // tile read before the next one overwrites it
+        for (int u = lane; u * 4 < pair * 16 * W; u += 64)
+            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, kStoreAux);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");    // tiles read before the next pair overwrites them
         __builtin_amdgcn_wave_barrier();
     }
 }
@@ -288,7 +290,7 @@ template <class DT, int C, int NBV>
 int launch_qk_n(float *attn, const void *a, const void *b, const Geom &g, const BandCover &c, hipStream_t s) {
     auto lds_of = [&](int nt) {
         return (size_t)region_bytes<C>(nt - 1 + NBV + ((c.shift & 15) ? 1 : 0)) + region_bytes<C>(nt) +
-               (size_t)kWaves * 16 * g.W * sizeof(float);
+               (size_t)kWaves * 32 * g.W * sizeof(float);
     };
     const int mt = fit_tiles(c.max_tiles, lds_of);
     if (mt < 1) return NA1D_ERR_UNSUPPORTED;
