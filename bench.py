@@ -360,6 +360,12 @@ def copy_yardstick(shapes, iters=100):
             total = (reads + writes) * nbytes
             out[label] = {"reads": reads, "writes": writes, "tensor_bytes": nbytes, "kernel_us": round(us, 3),
                           "GBps": round(total / us / 1e3, 1), "frac_of_hbm_peak": round(total / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            # the same copy with plain loads: the policy a kernel has to use for rows that another workgroup reads too
+            r = subprocess.run([exe, "copy", str(reads), str(writes), str(nbytes), str(iters), "plain"],
+                               capture_output=True, text=True, timeout=120)
+            m = re.search(r"copy_us=([0-9.]+)", r.stdout)
+            if r.returncode == 0 and m:
+                out[label]["plain_loads_kernel_us"] = round(float(m.group(1)), 3)
         except Exception as e:
             out[label] = {"error": "%s: %s" % (type(e).__name__, str(e)[:200])}
     return out

@@ -222,7 +222,9 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kCopyThreads = 256;
 // EPT 16-byte elements per thread and tensor: 4 KB, 8 KB or 16 KB per workgroup and tensor.  Which is fastest depends
 // on the launch size (small launches want many small workgroups), so the yardstick is the best of the three.
-template <int NR, int NW, int EPT>
+// NTL: the loads carry the non-temporal (read-once) policy; without it they are plain loads, the policy the operator's
+// strip copies have to use for rows that a neighbouring strip reads too.
+template <int NR, int NW, int EPT, bool NTL>
 __global__ void __launch_bounds__(kCopyThreads) copy_kernel(u32x4 *const *__restrict__ bufs, size_t n) {
     const size_t base = (size_t)blockIdx.x * EPT * kCopyThreads + threadIdx.x;
     u32x4 acc[EPT];
@@ -233,7 +235,7 @@ __global__ void __launch_bounds__(kCopyThreads) copy_kernel(u32x4 *const *__rest
 #pragma unroll
         for (int e = 0; e < EPT; ++e) {
             const size_t i = base + (size_t)e * kCopyThreads;
-            if (i < n) acc[e] ^= __builtin_nontemporal_load(&bufs[r][i]);      // read once: non-temporal
+            if (i < n) acc[e] ^= NTL ? __builtin_nontemporal_load(&bufs[r][i]) : bufs[r][i];
         }
 #pragma unroll
     for (int w = 0; w < NW; ++w)
@@ -247,15 +249,15 @@ __global__ void __launch_bounds__(kCopyThreads) copy_kernel(u32x4 *const *__rest
 
 // Average kernel time in us of `iters` launches, every launch between its own pair of events recorded by the launch
 // itself (the dispatch's begin and end), buffers rotated over `sets` sets.
-template <int NR, int NW, int EPT> double time_copy_variant(const std::vector<u32x4 **> &dsets, size_t n, int iters) {
+template <int NR, int NW, int EPT, bool NTL> double time_copy_variant(const std::vector<u32x4 **> &dsets, size_t n, int iters) {
     const int sets = (int)dsets.size();
     const unsigned grid = (unsigned)((n + kCopyThreads * EPT - 1) / (kCopyThreads * EPT));
-    for (int it = 0; it < sets + 3; ++it) copy_kernel<NR, NW, EPT><<<grid, kCopyThreads>>>(dsets[it % sets], n);
+    for (int it = 0; it < sets + 3; ++it) copy_kernel<NR, NW, EPT, NTL><<<grid, kCopyThreads>>>(dsets[it % sets], n);
     HIP_OK(hipDeviceSynchronize());
     std::vector<hipEvent_t> ev(2 * (size_t)iters);
     for (auto &e : ev) HIP_OK(hipEventCreate(&e));
     for (int it = 0; it < iters; ++it)
-        hipExtLaunchKernelGGL((copy_kernel<NR, NW, EPT>), dim3(grid), dim3(kCopyThreads), 0, nullptr, ev[2 * it],
+        hipExtLaunchKernelGGL((copy_kernel<NR, NW, EPT, NTL>), dim3(grid), dim3(kCopyThreads), 0, nullptr, ev[2 * it],
                               ev[2 * it + 1], 0, dsets[it % sets], n);
     HIP_OK(hipDeviceSynchronize());
     double total = 0;
@@ -268,7 +270,7 @@ template <int NR, int NW, int EPT> double time_copy_variant(const std::vector<u3
     return total * 1e3 / iters;
 }
 
-template <int NR, int NW> int time_copy(size_t bytes, int iters) {
+template <int NR, int NW, bool NTL> int time_copy(size_t bytes, int iters) {
     const size_t n = bytes / 16;
     const int nb = NR + NW, sets = (int)std::min(64.0, 700e6 / ((double)nb * (double)bytes) + 2);
     std::vector<u32x4 **> dsets;
@@ -283,26 +285,28 @@ template <int NR, int NW> int time_copy(size_t bytes, int iters) {
         HIP_OK(hipMemcpy(d, h.data(), nb * sizeof(void *), hipMemcpyHostToDevice));
         dsets.push_back(d);
     }
-    const double t1 = time_copy_variant<NR, NW, 1>(dsets, n, iters), t2 = time_copy_variant<NR, NW, 2>(dsets, n, iters),
-                 t4 = time_copy_variant<NR, NW, 4>(dsets, n, iters);
+    const double t1 = time_copy_variant<NR, NW, 1, NTL>(dsets, n, iters), t2 = time_copy_variant<NR, NW, 2, NTL>(dsets, n, iters),
+                 t4 = time_copy_variant<NR, NW, 4, NTL>(dsets, n, iters);
     const double us = std::min(t1, std::min(t2, t4));
-    std::printf("copy %dR+%dW x %zu bytes, %d launches: copy_us=%.3f GBps=%.1f (per thread and tensor 1 / 2 / 4 x 16 B: "
-                "%.3f / %.3f / %.3f us)\n", NR, NW, bytes, iters, us, (double)nb * (double)bytes / us / 1e3, t1, t2, t4);
+    std::printf("copy %dR+%dW x %zu bytes, %s loads, %d launches: copy_us=%.3f GBps=%.1f (per thread and tensor 1 / 2 / 4 x 16 B: "
+                "%.3f / %.3f / %.3f us)\n", NR, NW, bytes, NTL ? "read-once" : "plain", iters, us,
+                (double)nb * (double)bytes / us / 1e3, t1, t2, t4);
     return 0;
 }
 
 int copy_mode(int argc, char **argv) {
-    if (argc != 6) {
-        std::printf("usage: %s copy READS WRITES BYTES ITERS\n", argv[0]);
+    if (argc != 6 && !(argc == 7 && std::strcmp(argv[6], "plain") == 0)) {
+        std::printf("usage: %s copy READS WRITES BYTES ITERS [plain]   (plain: loads without the read-once policy)\n", argv[0]);
         return 64;
     }
+    const bool plain = argc == 7;
     const int r = std::atoi(argv[2]), w = std::atoi(argv[3]), iters = std::atoi(argv[5]);
     const size_t bytes = (size_t)std::atoll(argv[4]) / 16 * 16;
     if (iters < 1 || iters > 10000 || bytes < 16 || bytes > ((size_t)1 << 31)) return 64;
-    if (r == 3 && w == 1) return time_copy<3, 1>(bytes, iters);
-    if (r == 4 && w == 3) return time_copy<4, 3>(bytes, iters);
-    if (r == 2 && w == 1) return time_copy<2, 1>(bytes, iters);
-    if (r == 1 && w == 1) return time_copy<1, 1>(bytes, iters);
+    if (r == 3 && w == 1) return plain ? time_copy<3, 1, false>(bytes, iters) : time_copy<3, 1, true>(bytes, iters);
+    if (r == 4 && w == 3) return plain ? time_copy<4, 3, false>(bytes, iters) : time_copy<4, 3, true>(bytes, iters);
+    if (r == 2 && w == 1) return plain ? time_copy<2, 1, false>(bytes, iters) : time_copy<2, 1, true>(bytes, iters);
+    if (r == 1 && w == 1) return plain ? time_copy<1, 1, false>(bytes, iters) : time_copy<1, 1, true>(bytes, iters);
     std::printf("copy: READS+WRITES must be 1+1, 2+1, 3+1 or 4+3\n");
     return 64;
 }
