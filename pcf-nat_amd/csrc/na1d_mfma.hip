@@ -326,6 +326,7 @@ drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, 
 #define NA1D_BWD_MIN_WAVES(C, DROP) ((C) == 16 && !(DROP) ? 6 : 1)
 #endif
 
+constexpr int kBwdMinItems = 256;      // fewer items than this: shorter strips
 template <int C> struct StripBwd {
 #ifdef NA1D_BWD_MT
     static constexpr int kMaxTiles = NA1D_BWD_MT * 32 / (C < 32 ? 32 : C);
@@ -653,7 +654,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                const void *dout, const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g,
                const Layout &in, const Layout &outl, float scale, float *workspace, int64_t workspace_bytes,
                hipStream_t s) {
-    const Split sp = make_split(g.B, g.T, StripBwd<C>::kMaxTiles);
+    const Split sp = make_split(g.B, g.T, StripBwd<C>::kMaxTiles, kBwdMinItems);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
     float *partial = nullptr;
     if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
@@ -678,7 +679,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
 
 template <class DT, int C>
 int64_t bwd_workspace(const Geom &g) {
-    return make_split(g.B, g.T, StripBwd<C>::kMaxTiles).items * kPartialStride * (int64_t)sizeof(float);
+    return make_split(g.B, g.T, StripBwd<C>::kMaxTiles, kBwdMinItems).items * kPartialStride * (int64_t)sizeof(float);
 }
 
 int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,

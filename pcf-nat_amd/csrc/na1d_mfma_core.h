@@ -369,12 +369,13 @@ struct Split {
     int strips;      // strips per sequence
     int64_t items;   // workgroups
 };
-inline Split make_split(int64_t B, int64_t T, int max_tiles) {
+inline Split make_split(int64_t B, int64_t T, int max_tiles, int min_items = 1024) {
     Split s;
     s.tiles = (int)((T + 15) / 16);
     s.strips = (s.tiles + max_tiles - 1) / max_tiles;
-    // small problems: more, shorter strips so that every CU gets a few workgroups
-    while (B * s.strips < 1024 && s.strips < s.tiles) ++s.strips;
+    // small problems: more, shorter strips so that every CU gets a few workgroups (the backward, whose strips carry
+    // a halo of query tiles, is better off with one workgroup per CU and longer strips)
+    while (B * s.strips < min_items && s.strips < s.tiles) ++s.strips;
     s.nt = (s.tiles + s.strips - 1) / s.strips;
     s.strips = (s.tiles + s.nt - 1) / s.nt;
     s.items = B * s.strips;
