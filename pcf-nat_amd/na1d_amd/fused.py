@@ -183,8 +183,9 @@ class _FusedNA1DQKV(torch.autograd.Function):
     """Fused NA1D straight on the qkv projection's output ``[N, T, 3, H, C]`` -> ``[N, T, H*C]``."""
 
     @staticmethod
-    def forward(ctx, qkv, rpb, t_valid, win_size, left, scale, deterministic, dilation):
+    def forward(ctx, qkv, rpb, t_valid, win_size, left, scale, deterministic, dilation, dropout):
         assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.is_contiguous() and dilation >= 1
+        ctx.dropout = dropout
         N, T, _, H, C = qkv.shape
         ctx.rpb_shape = None if rpb is None else rpb.shape
         if rpb is not None:
@@ -201,7 +202,8 @@ class _FusedNA1DQKV(torch.autograd.Function):
             lse = torch.empty((N * H, qr.shape[2]), dtype=torch.float32, device=qkv.device)
             ctx.packed_outs.append(_strided_or_packed_forward(
                 _residue(o4, r, dilation), lse, qr, _residue(k4, r, dilation), _residue(v4, r, dilation), rpb,
-                _residue_lengths(t_valid, r, dilation), win_size, left, scale))
+                _residue_lengths(t_valid, r, dilation), win_size, left, scale,
+                dropout=None if dropout is None else (*dropout, dilation, r, T)))
             lses.append(lse)
         ctx.save_for_backward(qkv, rpb, t_valid, *lses)
         ctx.geom = (win_size, left, scale, deterministic, dilation)
@@ -224,13 +226,15 @@ class _FusedNA1DQKV(torch.autograd.Function):
             a = [_residue(z, r, dilation) for z in views]
             _strided_or_packed_backward(a[0], a[1], a[2], drpb, a[3], a[4], a[5], ctx.packed_outs[r],
                                         _residue(g4, r, dilation), lse, rpb, _residue_lengths(t_valid, r, dilation),
-                                        win_size, left, scale, ws)
+                                        win_size, left, scale, ws,
+                                        dropout=None if ctx.dropout is None else (*ctx.dropout, dilation, r, T))
         if drpb is not None:
             drpb = drpb.view(ctx.rpb_shape)
-        return dqkv, drpb, None, None, None, None, None, None
+        return dqkv, drpb, None, None, None, None, None, None, None
 
 
-def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deterministic=False, dilation=1):
+def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deterministic=False, dilation=1,
+                   dropout_p=0.0, seed=None):
     """Fused neighbourhood attention on a token-major qkv projection output.
 
     qkv : contiguous ``[N, T, 3, H, C]`` bf16/fp16 (the ``[N, T, 3*dim]`` output of the projection, viewed).
@@ -238,9 +242,16 @@ def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deter
           and merge copies of the reference (models/MFA_NATransformer.py:127-138,150-151) do not exist; the
           gradient comes back as one ``[N, T, 3, H, C]`` tensor.  ``scale`` multiplies the fp32 scores (the
           reference multiplies q by it in 16 bit beforehand).
-    Other arguments as in :func:`na1d_fused`.
+    Other arguments as in :func:`na1d_fused`; with ``dropout_p`` the mask is the one :func:`na1d_fused` draws for the
+    same seed on the split tensors (sequence n * H + h, row, slot).
     """
-    if dilation == 1 and not (torch.is_grad_enabled() and (qkv.requires_grad or (rpb is not None and rpb.requires_grad))):
+    dropout = None
+    if dropout_p > 0.0:
+        assert dropout_p < 1.0
+        if seed is None:
+            seed = int(torch.randint(0, 2 ** 62, (1,)).item())
+        dropout = (float(dropout_p), int(seed))
+    if dropout is None and dilation == 1 and not (torch.is_grad_enabled() and (qkv.requires_grad or (rpb is not None and rpb.requires_grad))):
         # inference: one library call, no views, no log-sum-exp
         assert qkv.dim() == 5 and qkv.shape[2] == 3 and qkv.is_contiguous()
         N, T, _, H, C = qkv.shape
@@ -254,4 +265,5 @@ def na1d_fused_qkv(qkv, win_size, left, rpb=None, t_valid=None, scale=1.0, deter
         out = torch.empty((N, T, H * C), dtype=qkv.dtype, device=qkv.device)
         if N * T == 0 or _lib.call_fused_forward_qkv(out, None, qkv, rpb, t_valid, win_size, left, float(scale)) == 0:
             return out
-    return _FusedNA1DQKV.apply(qkv, rpb, t_valid, win_size, left, float(scale), bool(deterministic), int(dilation))
+    return _FusedNA1DQKV.apply(qkv, rpb, t_valid, win_size, left, float(scale), bool(deterministic), int(dilation),
+                               dropout)

@@ -405,8 +405,8 @@ class NAttention(nn.Module):
             padding = None
         t_valid = None if padding is None else (t - padding).to(torch.int32)
         dropping = self.attn_drop > 0.0 and self.training
-        if self.na == "fused_qkv" and not dropping:
-            return self.proj_drop(self._forward_token_major(x, n, t, t_valid))
+        if self.na == "fused_qkv":                           # dropout (PCF :149) happens inside the kernels
+            return self.proj_drop(self._forward_token_major(x, n, t, t_valid, self.attn_drop if dropping else 0.0))
         q, k, v = _split_heads(self.qkv(x), h, self.groups, self.channels_first)
         q = q * self.scale                                   # in the activation dtype, as the reference does (:141)
         extra = {} if self.dilation == 1 else {"dilation": self.dilation}
@@ -430,7 +430,7 @@ class NAttention(nn.Module):
             out = self.NA1d_AV_Function.apply(attn, v, w, left, 1)
         return self.proj_drop(self.proj(_merge_heads(out, n, h, self.channels_first)))
 
-    def _forward_token_major(self, x, n, t, t_valid):
+    def _forward_token_major(self, x, n, t, t_valid, dropout_p=0.0):
         """The same layer with the operator reading the qkv projection in place.  Tokens-first models have the
         layout already; channels-first ones get it by running the two 1x1 convolutions as matrix products whose
         output rows are ordered (which, head, channel) - the same parameters, the same arithmetic, no copies."""
@@ -444,7 +444,7 @@ class NAttention(nn.Module):
             qkv = self.qkv(x)
         out = na1d_fused_qkv(qkv.view(n, t, 3, h, self.dim // h), self.win_size, self.left,
                              rpb=self.relative_position_bias, t_valid=t_valid, scale=self.scale,
-                             dilation=self.dilation)                                                  # [N, T, dim]
+                             dilation=self.dilation, dropout_p=dropout_p)                             # [N, T, dim]
         if self.channels_first:
             wp, bp = _prepared(self.proj, "dense", out, lambda: (_dense_weight(self.proj), self.proj.bias))
             return torch.bmm(wp.unsqueeze(0).expand(n, -1, -1), out.transpose(1, 2)).add_(bp.view(1, -1, 1))  # [N, dim, T]

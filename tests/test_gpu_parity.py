@@ -687,6 +687,30 @@ def test_strided_dropout_rejects_rows_outside_the_sequence():
             _lib.call_fused_forward_strided(torch.empty_like(q), lse, q, q, q, None, None, 5, 2, 1.0, dropout=bad)
 
 
+@pytest.mark.parametrize("dilation", [1, 2])
+def test_in_place_qkv_operator_drops_like_the_split_one(dilation):
+    """na1d_fused_qkv(..., dropout_p, seed) on [N, T, 3, H, C] draws the mask na1d_fused draws on the split tensors
+    (sequence n * H + h), forward and backward."""
+    N, H, T, C, W, L, p, seed = 2, 4, 90, 16, 27, 13, 0.25, 1234567
+    g = torch.Generator().manual_seed(8)
+    qkv = (torch.randn(N, T, 3, H, C, generator=g) * 0.5).to(torch.float16).cuda().requires_grad_(True)
+    rpb = (torch.randn(H, W, generator=g) * 0.3).cuda().requires_grad_(True)
+    t_valid = torch.tensor([T, T - 17], dtype=torch.int32).cuda()
+    do = torch.randn(N, T, H * C, generator=g).to(torch.float16).cuda()
+    out = na1d_fused_qkv(qkv, W, L, rpb=rpb, t_valid=t_valid, scale=1.0, dilation=dilation, dropout_p=p, seed=seed)
+    out.backward(do)
+    q, k, v = (qkv.detach()[:, :, i].permute(0, 2, 1, 3).reshape(N * H, T, C).contiguous().requires_grad_(True) for i in range(3))
+    rpb2 = rpb.detach().clone().requires_grad_(True)
+    ref = na1d_fused(q, k, v, W, L, rpb=rpb2, t_valid=t_valid, num_heads=H, dilation=dilation, dropout_p=p, seed=seed)
+    ref.backward(do.view(N, T, H, C).permute(0, 2, 1, 3).reshape(N * H, T, C))
+    assert torch.equal(out.view(N, T, H, C).permute(0, 2, 1, 3).reshape(N * H, T, C), ref)
+    for i, z in enumerate((q, k, v)):
+        assert torch.equal(qkv.grad[:, :, i].permute(0, 2, 1, 3).reshape(N * H, T, C), z.grad)
+    assert torch.allclose(rpb.grad, rpb2.grad, rtol=1e-4, atol=1e-5)
+    plain = na1d_fused_qkv(qkv.detach(), W, L, rpb=rpb.detach(), t_valid=t_valid, dilation=dilation)
+    assert not torch.equal(plain, out.detach())
+
+
 def test_dropout_rate_zero_is_the_plain_operator_and_bad_rates_are_rejected():
     q, k, v = dev(*make_inputs(4, 50, 32, 15, 3, torch.bfloat16))
     assert torch.equal(na1d_fused(q, k, v, 15, 7, dropout_p=0.0), na1d_fused(q, k, v, 15, 7))
