@@ -340,8 +340,8 @@ global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__re
         if (c0) __syncthreads();
         stage_direct<C, kStripTiles, kReadShared>(qs, 16 * c0, q_lds, kStripTiles, wave, lane_off, a.pitch);
         stage_direct<C, kStripTiles, kReadShared>(gs, 16 * c0, g_lds, kStripTiles, wave, lane_off, a.pitch);
-        if (wave == 0) __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))lse_lds, 4, (16 * c0 + lane) * 4, 0, 0, 0);
-        if (wave == 1) __builtin_amdgcn_raw_ptr_buffer_load_lds(ds, (LDS_PTR(void))del_lds, 4, (16 * c0 + lane) * 4, 0, 0, 0);
+        if (wave == 0) load_to_lds<4, 0>(ls, (LDS_PTR(char))lse_lds, (16 * c0 + lane) * 4);
+        if (wave == 1) load_to_lds<4, 0>(ds, (LDS_PTR(char))del_lds, (16 * c0 + lane) * 4);
         wait_direct();
         __syncthreads();
         if (c0 == 0) {

@@ -69,84 +69,114 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     const bool out_whole_lines = stores_whole_lines(outl.pitch, C, 0);
     const bool out_grouped = HG > 1 && outl.head == 2 * C && outl.width == 2 * C && outl.pitch >= HG * 2 * C;
 
-    // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
-    {
-        const int lane_off = direct_lane_offset<CS>(wave, lane, in.pitch, HG * in.width);
-        const bool whole_lines = in.pitch == 2 * C || CS % 64 == 0;
-        if (strips == 1 && whole_lines) {      // nobody else reads these rows' lines
-            stage_direct<CS, MT + 2, kReadOnce, NW>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
-            stage_direct<CS, MT, kReadOnce, NW>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-            stage_direct<CS, MT + 2, kReadOnce, NW>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
-        } else {
-            stage_direct<CS, MT + 2, kReadShared, NW>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
-            if (whole_lines)
-                stage_direct<CS, MT, kReadOnce, NW>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-            else
-                stage_direct<CS, MT, kReadShared, NW>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
-            stage_direct<CS, MT + 2, kReadShared, NW>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
-        }
-    }
-
     BiasTable bias_raw;
     load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
 
+    // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
+    constexpr int TW = NW / HG;                      // tiles the workgroup computes side by side
+    {
+        const int lane_off = direct_lane_offset<CS>(wave, lane, in.pitch, HG * in.width);
+        const bool whole_lines = in.pitch == 2 * C || CS % 64 == 0;
+        auto stage = [&](auto key_aux, auto qry_aux) {
+            constexpr int KA = decltype(key_aux)::value, QA = decltype(qry_aux)::value;
+            stage_direct<CS, MT + 2, KA, NW>(ks, 16 * i0 - 16, k_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<CS, MT, QA, NW>(qs, 16 * i0, q_lds, nt, wave, lane_off, in.pitch);
+            stage_direct<CS, MT + 2, KA, NW>(vs, 16 * i0 - 16, v_lds, nt + 2, wave, lane_off, in.pitch);
+        };
+        using Once = std::integral_constant<int, kReadOnce>;
+        using Shared = std::integral_constant<int, kReadShared>;
+        if (strips == 1 && whole_lines)         // nobody else reads these rows' lines
+            stage(Once{}, Once{});
+        else if (whole_lines)
+            stage(Shared{}, Once{});
+        else
+            stage(Shared{}, Shared{});
+    }
+
     int tv = T;
-    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    if (t_valid) tv = max(0, min(T, load_uniform_i32(t_valid, sample)));
+    // The matrix core adds the bias for nothing: accumulators start at rpb / scale (-inf outside the window), so
+    // x = q.k + rpb / scale comes out of the instruction, z = x * scale * log2(e) is the logit in the log2 domain,
+    // and exp2(z - max z) is one multiply-add per slot on the way into the exponential (scale > 0).
     const float scale2 = scale * kLog2e;
+    const float inv_scale = __builtin_amdgcn_rcpf(scale);
 
     // per-lane LDS offsets; key-side regions start 16 rows before the strip
+    const int slot = wave / HG;
     RowLane<C, CS> k_lane, q_lane;
     TrLane<C, CS> v_lane;
     k_lane.init(16 - shift, lane, hw * 2 * C);
     q_lane.init(0, lane, hw * 2 * C);
     v_lane.init(16 - shift, lane, hw * 2 * C);
+    LDS_PTR(char) k_mine = k_lds + slot * LL::kTileBytes;      // this wave's first tile in each region
+    LDS_PTR(char) v_mine = v_lds + slot * LL::kTileBytes;
+    LDS_PTR(char) q_mine = q_lds + slot * LL::kTileBytes;
 
     const uint32_t one2 = DT::tag == NA1D_BF16 ? 0x3f803f80u : 0x3c003c00u;
     const u32x2 ones = {one2, one2};                 // a 16 x 16 block of ones as a matrix operand
+    // everything that depends on the lane alone is worked out while the copies are in flight
+#pragma unroll
+    for (int s_ = 0; s_ < (RowOperand<C>::k32 > 0 ? RowOperand<C>::k32 : 1); ++s_) {
+        settle(k_lane.off32[s_]);
+        settle(q_lane.off32[s_]);
+    }
+    settle(k_lane.off16);
+    settle(q_lane.off16);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) settle(v_lane.off[ct]);
 
     wait_direct();
-    write_bias_table(bias_lds, bias_raw, W, lane);
+    wait_bias(bias_raw);
+    write_bias_table(bias_lds, bias_raw, W, lane, inv_scale);
     Window<NBV> win;
     read_window<NBV>(win, bias_lds, L, shift, g, n);
-    __syncthreads();
+    barrier_lds();
 
-    for (int i = i0 + wave / HG; i < i1; i += NW / HG) {
-        const int tile_bytes = (i - i0) * LL::kTileBytes;
+    const f32x4 bias_x = {win.bias_x[0], win.bias_x[1], win.bias_x[2], win.bias_x[3]};
+    const f32x4 bias_y = {win.bias_y[0], win.bias_y[1], win.bias_y[2], win.bias_y[3]};
+    const float mask_x = kMaskValue * inv_scale;     // the model's additive -100, before the scale
+    const int strip_tiles = i1 - i0;
+#pragma unroll
+    for (int jt = 0; jt < (MT + TW - 1) / TW; ++jt) {
+        const int li = slot + jt * TW;               // tile inside the strip
+        if (li >= strip_tiles) break;
+        const int i = i0 + li;
+        const int tile_bytes = jt * TW * LL::kTileBytes;         // behind this wave's first tile: a constant
         RowOperand<C> qt;
-        read_rows<C>(qt, q_lds + tile_bytes, q_lane);
+        read_rows<C>(qt, q_mine + tile_bytes, q_lane);
 
-        // S^T for the virtual key blocks
+        // x^T = bias + K . Q^T for the virtual key blocks
         f32x4 s[NBV];
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
             RowOperand<C> kop;
-            read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
-            s[vb] = dot_rows_mma<DT, C>(kop, qt);
+            read_rows<C>(kop, k_mine + tile_bytes + vb * LL::kTileBytes, k_lane);
+            s[vb] = dot_rows_mma<DT, C>(kop, qt, vb == 1 ? bias_y : bias_x);
         }
         float zx[4], zy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[NBV - 1][r]) : s[0][r];
-            zx[r] = __builtin_fmaf(sx, scale2, win.bias_x[r]);
-            zy[r] = __builtin_fmaf(s[1][r], scale2, win.bias_y[r]);
+            zx[r] = NBV == 3 ? (win.from0[r] ? s[0][r] : s[NBV - 1][r]) : s[0][r];
+            zy[r] = s[1][r];
         }
 
         // additive -100 of the model's mask, only on tiles that touch an edge
         const int s0 = 16 * i - shift;           // first row of the window
         const int qrow = 16 * i + n;
         if (s0 < 0 || s0 + 16 * NBV > tv) {
-            const bool row_masked = qrow >= tv;  // a padded query row masks all of its slots
+            const uint32_t tve = qrow >= tv ? 0u : (uint32_t)tv;     // a padded query row masks all of its slots
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const uint32_t key_y = (uint32_t)(s0 + 16 + 4 * g + r);
                 const uint32_t key_x = (uint32_t)(s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0));
-                zx[r] += (key_x >= (uint32_t)tv || row_masked) ? kMaskValue * kLog2e : 0.f;   // unsigned: also key < 0
-                zy[r] += (key_y >= (uint32_t)tv || row_masked) ? kMaskValue * kLog2e : 0.f;
+                zx[r] += key_x >= tve ? mask_x : 0.f;   // unsigned: also key < 0
+                zy[r] += key_y >= tve ? mask_x : 0.f;
             }
         }
 
         float m = max3(max3(zx[0], zx[1], zx[2]), max3(zx[3], zy[0], zy[1]), max2(zy[2], zy[3]));
         m = xor_max(m);
+        const float nm = -m * scale2;
 
         // The row sums that normalise the output come from the matrix core: a product of the rounded probabilities
         // with a block of ones leaves every lane the sum of its query's row (what the output's numerator was
@@ -157,8 +187,8 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         float px[4], py[4], sum = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            px[r] = __builtin_amdgcn_exp2f(zx[r] - m);
-            py[r] = __builtin_amdgcn_exp2f(zy[r] - m);
+            px[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(zx[r], scale2, nm));
+            py[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(zy[r], scale2, nm));
         }
         if (!kMmaSum || lse) {
 #pragma unroll
@@ -192,7 +222,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int vb = 0; vb < NBV; ++vb) {
-            LDS_PTR(char) blk = v_lds + tile_bytes + vb * LL::kTileBytes;
+            LDS_PTR(char) blk = v_mine + tile_bytes + vb * LL::kTileBytes;
             if constexpr (kMmaSum) rowsum = Mma<DT>::k16(ones, pb[vb], rowsum);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr(blk + v_lane.off[ct]), pb[vb], o[ct]);
@@ -203,22 +233,21 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
+        const float lse_row = (__builtin_amdgcn_logf(sum) - nm) * kLn2;
         if (HG > 1 && out_grouped) {          // into the place of this head's Q tile, which only this wave has read
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct)
-                *reinterpret_cast<LDS_PTR(u32x2)>(q_lds + tile_bytes + LL::addr(n, hw * 2 * C + 32 * ct + 8 * g)) = ow[ct];
+                *reinterpret_cast<LDS_PTR(u32x2)>(q_mine + tile_bytes + LL::addr(n, hw * 2 * C + 32 * ct + 8 * g)) = ow[ct];
         } else {
             store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines, outl.width);
         }
-        if (g == 0)
-            __builtin_amdgcn_raw_buffer_store_b32(
-                __float_as_uint((m + __builtin_amdgcn_logf(sum)) * kLn2), ls, qrow * 4, 0, 0);
+        if (lse && g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(lse_row), ls, qrow * 4, 0, 0);
     }
     if (HG > 1 && out_grouped) {
         // The heads of a group lie side by side in the output too: the strip's output rows, collected in the Q
         // region, leave as whole lines - the strip copy run backwards, each lane taking the 16-byte unit that sits
         // at its place in LDS to where it belongs in memory.
-        __syncthreads();
+        barrier_lds();
         constexpr int kRounds = (region_bytes<CS>(MT) / kChunk + NW - 1) / NW;
         constexpr int kChunkRows = kChunk / LL::kRowBytes;
         const Rsrc gs = make_rsrc(out + sample * outl.sample + head0 * outl.head, min(T, 16 * i1) * outl.pitch);
@@ -326,6 +355,10 @@ drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, 
 #define NA1D_BWD_MIN_WAVES(C, DROP) ((C) == 16 && !(DROP) ? 6 : 1)
 #endif
 
+// Rows that no other workgroup reads: the backward takes them with the workgroup-scope policy rather than the
+// non-temporal one of the forward (measured: 4-7 % on the 16-channel backward, nothing either way at 32 channels; the
+// forward loses 3-8 % with it).
+constexpr int kReadOnceBwd = 1;
 constexpr int kBwdMinItems = 256;      // fewer items than this: shorter strips
 template <int C> struct StripBwd {
 #ifdef NA1D_BWD_MT
@@ -378,6 +411,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     const int sc_skip = strips == 1 ? 1 : 0;       // a strip that is the whole sequence has no halo tiles to keep scores of
 
     const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
+    BiasTable bias_raw;
+    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
     {
         const int key_bytes = min(T, 16 * (i1 + 2)) * in.pitch;
         const int qry_rows = min(T, 16 * (i1 + 1));
@@ -387,12 +422,12 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
         const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch, outl.width);
         // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * i0 - 16 + tid) * 4, 0, 0, 0);
+        load_to_lds<4, 0>(ls, (LDS_PTR(char))(lse_lds + 64 * wave), (16 * i0 - 16 + tid) * 4);
         if (strips == 1 && (in.pitch == 2 * C || C % 64 == 0) && (outl.pitch == 2 * C || C % 64 == 0)) {
-            stage_direct<C, MT + 1 + NBV, kReadOnce>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadOnce>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 1 + NBV, kReadOnce>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadOnce>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
+            stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadOnceBwd>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2, kReadOnceBwd>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
         } else {
             stage_direct<C, MT + 1 + NBV, kReadShared>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
             stage_direct<C, MT + 2, kReadShared>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
@@ -401,13 +436,12 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
 
-    BiasTable bias_raw;
-    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
-
     int tv = T;
-    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    if (t_valid) tv = max(0, min(T, load_uniform_i32(t_valid, sample)));
+    // as in the forward: the accumulators start at rpb / scale, z = x * scale * log2(e) - lse is one multiply-add
     const float scale2 = scale * kLog2e;
-    const float mask2 = kMaskValue * kLog2e;
+    const float inv_scale = __builtin_amdgcn_rcpf(scale);
+    const float mask_x = kMaskValue * inv_scale;
 
     RowLane<C> key_lane, qry_lane;      // row operands: virtual key block rows / query tile rows
     TrLane<C> key_tr, qry_tr;           // transposed operands of the same
@@ -415,12 +449,28 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     key_tr.init(0, lane);
     qry_lane.init(0, lane);
     qry_tr.init(0, lane);
+    // everything that depends on the lane alone is worked out while the copies are in flight
+#pragma unroll
+    for (int s_ = 0; s_ < (RowOperand<C>::k32 > 0 ? RowOperand<C>::k32 : 1); ++s_) {
+        settle(key_lane.off32[s_]);
+        settle(qry_lane.off32[s_]);
+    }
+    settle(key_lane.off16);
+    settle(qry_lane.off16);
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        settle(key_tr.off[ct]);
+        settle(qry_tr.off[ct]);
+    }
 
     wait_direct();
-    write_bias_table(bias_lds, bias_raw, W, lane);
+    wait_bias(bias_raw);
+    write_bias_table(bias_lds, bias_raw, W, lane, inv_scale);
     Window<NBV> win;
     read_window<NBV>(win, bias_lds, L, shift, g, n);
-    __syncthreads();
+    barrier_lds();
+    const f32x4 bias_x = {win.bias_x[0], win.bias_x[1], win.bias_x[2], win.bias_x[3]};
+    const f32x4 bias_y = {win.bias_y[0], win.bias_y[1], win.bias_y[2], win.bias_y[3]};
 
     // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
@@ -443,35 +493,35 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             const int off = (qt - i0 + 1 + vb) * LL::kTileBytes;
             read_rows<C>(kop, k_lds + off, key_lane);
             read_rows<C>(vop, v_lds + off, key_lane);
-            s[vb] = dot_rows_mma<DT, C>(kop, qop);
+            s[vb] = dot_rows_mma<DT, C>(kop, qop, vb == 1 ? bias_y : bias_x);
             dp[vb] = dot_rows_mma<DT, C>(vop, gop);
         }
-        const float lse2 = lse_lds[tq * 16 + n] * kLog2e;
+        const float nlse2 = -lse_lds[tq * 16 + n] * kLog2e;
         float zx[4], zy[4], dpx[4], dpy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float sx = NBV == 3 ? (win.from0[r] ? s[0][r] : s[NBV - 1][r]) : s[0][r];
+            zx[r] = NBV == 3 ? (win.from0[r] ? s[0][r] : s[NBV - 1][r]) : s[0][r];
             dpx[r] = NBV == 3 ? (win.from0[r] ? dp[0][r] : dp[NBV - 1][r]) : dp[0][r];
             dpy[r] = dp[1][r];
-            zx[r] = __builtin_fmaf(sx, scale2, win.bias_x[r]) - lse2;
-            zy[r] = __builtin_fmaf(s[1][r], scale2, win.bias_y[r]) - lse2;
+            zy[r] = s[1][r];
         }
         const int s0 = 16 * qt - shift;
         const int qrow = 16 * qt + n;
         if (s0 < 0 || s0 + 16 * NBV > tv) {
+            const uint32_t tve = qrow >= tv ? 0u : (uint32_t)tv;     // a padded query row masks all of its slots
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const uint32_t key_y = (uint32_t)(s0 + 16 + 4 * g + r);
                 const uint32_t key_x = (uint32_t)(s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0));
-                zx[r] += (key_x >= (uint32_t)tv || qrow >= tv) ? mask2 : 0.f;   // unsigned: also key < 0
-                zy[r] += (key_y >= (uint32_t)tv || qrow >= tv) ? mask2 : 0.f;
+                zx[r] += key_x >= tve ? mask_x : 0.f;   // unsigned: also key < 0
+                zy[r] += key_y >= tve ? mask_x : 0.f;
             }
         }
         float px[4], py[4], part = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            px[r] = __builtin_amdgcn_exp2f(zx[r]);
-            py[r] = __builtin_amdgcn_exp2f(zy[r]);
+            px[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(zx[r], scale2, nlse2));
+            py[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(zy[r], scale2, nlse2));
         }
         // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dV takes D*P and dP = D * (dO . V^T).
         float fx[4] = {1.f, 1.f, 1.f, 1.f}, fy[4] = {1.f, 1.f, 1.f, 1.f};
@@ -563,7 +613,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         if (g == 1) rsum[wave * 32 + ((slot + 16) & 31)] = s1;
     }
 
-    __syncthreads();                    // every wave is done with K and V: their regions become the score tiles
+    barrier_lds();                    // every wave is done with K and V: their regions become the score tiles
 #pragma unroll
     for (int jt = 0; jt < TPW; ++jt) {
         const int tq = wave + jt * kWaves;
@@ -575,7 +625,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 #pragma unroll
             for (int pd = 0; pd < 2; ++pd) *reinterpret_cast<LDS_PTR(u32x2)>(t + (xy * 2 + pd) * kScoreTile) = sc[jt][xy][pd];
     }
-    __syncthreads();
+    barrier_lds();
 
     // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
     // key block kp covers rows 16*kp - shift .. +15 and is virtual block vb of query tile kp - vb.  Lane (n, g)
@@ -638,7 +688,9 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         store_tile<C>(dvs, row_off, vw, g, whole_lines, in.width);
     }
 
-    if (drpb && tid < W) {              // rsum was complete at the barriers before pass 2
+    // last, behind the gradient stores: issued earlier (the sums are complete before pass 2) the atomics cost the
+    // kernel twice as much, the stores of pass 2 queueing behind them
+    if (drpb && tid < W) {
         float t = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) t += rsum[w * 32 + tid];

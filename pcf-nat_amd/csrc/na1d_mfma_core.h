@@ -38,6 +38,7 @@
 
 #include <algorithm>
 #include <cstdio>
+#include <type_traits>
 
 #include <hip/hip_ext.h>
 
@@ -167,6 +168,24 @@ __device__ inline int direct_lane_offset(int wave, int lane, int pitch = Lds<C>:
     const int unit = su ^ Lds<C>::swz(u / Lds<C>::kUnits);
     return unit * 16 < width ? (lane / Lds<C>::kUnits) * pitch + unit * 16 : kNowhere;
 }
+// One wave-wide load that writes LDS directly: lane l's BYTES (4 or 16) land at lds + BYTES * l.  Written out by hand
+// so that the compiler knows nothing of it: told of such loads it puts waits for ALL of them in front of LDS reads it
+// cannot tell apart from their target, which defeats copies that are issued early and waited for in parts.  Callers
+// wait with wait_direct() before they (or, behind a barrier, other waves) read the target.
+template <int BYTES, int AUX>
+__device__ inline void load_to_lds(Rsrc src, LDS_PTR(char) lds, int offset) {
+    static_assert((BYTES == 4 || BYTES == 16) && (AUX == 0 || AUX == 1 || AUX == 2 || AUX == 3), "load size / cache policy");
+    const uint32_t at = __builtin_amdgcn_readfirstlane((uint32_t)reinterpret_cast<uintptr_t>(lds));      // wave-uniform by contract
+    if constexpr (BYTES == 16) {
+        if constexpr (AUX == 0) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(at), "v"(offset), "s"(src) : "memory");
+        if constexpr (AUX == 1) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen sc0 lds" ::"s"(at), "v"(offset), "s"(src) : "memory");
+        if constexpr (AUX == 2) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds" ::"s"(at), "v"(offset), "s"(src) : "memory");
+        if constexpr (AUX == 3) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen sc0 nt lds" ::"s"(at), "v"(offset), "s"(src) : "memory");
+    } else {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds" ::"s"(at), "v"(offset), "s"(src) : "memory");
+    }
+}
+
 template <int C, int NTILES, int AUX, int NW = kWaves>       // NW: the waves of the workgroup that share the copy
 __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, int ntiles, int wave, int lane_off,
                                     int pitch = Lds<C>::kRowBytes) {
@@ -178,11 +197,17 @@ __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, 
 #pragma unroll
     for (int j = 0; j < kRounds; ++j) {
         const int c = j * NW + wave;
-        if (c < chunks)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * kChunk), 16, base + c * step, 0, 0, AUX);
+        if (c < chunks) load_to_lds<16, AUX>(src, region + c * kChunk, base + c * step);
     }
 }
 __device__ inline void wait_direct() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// Workgroup barrier that waits for this wave's LDS accesses only.  __syncthreads() also waits for every vector-memory
+// access in flight, i.e. for strip copies that were issued early on purpose; what has to have landed is waited for
+// explicitly (wait_direct) in front of this.
+__device__ inline void barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// Have a value worked out here rather than where it is first used: per-lane constants placed in front of the wait for
+// the strip copies cost nothing, behind it they delay the first tile.
+template <class T> __device__ inline void settle(T &x) { asm volatile("" : "+v"(x)); }
 
 // ---- operands out of LDS ------------------------------------------------------
 // Row operand (A or B of a contraction over channels): lane (n, g) holds row n of a
@@ -213,8 +238,7 @@ __device__ inline void read_rows(RowOperand<C> &o, LDS_PTR(char) tile, const Row
     if (RowOperand<C>::k16) o.w16[0] = *reinterpret_cast<LDS_PTR(u32x2)>(tile + l.off16);
 }
 template <class DT, int C>
-__device__ inline f32x4 dot_rows_mma(const RowOperand<C> &a, const RowOperand<C> &b) {
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+__device__ inline f32x4 dot_rows_mma(const RowOperand<C> &a, const RowOperand<C> &b, f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f}) {
 #pragma unroll
     for (int s = 0; s < RowOperand<C>::k32; ++s) acc = Mma<DT>::k32(a.w32[s], b.w32[s], acc);
     if (RowOperand<C>::k16) acc = Mma<DT>::k16(a.w16[0], b.w16[0], acc);
@@ -324,12 +348,19 @@ constexpr int kBiasPad = 32, kBiasEntries = 64;         // slots -32 .. 31 cover
 struct BiasTable {
     float raw;
 };
+// The load is written out by hand: the compiler, which cannot count the strip copies that follow it through their
+// branches, would otherwise put a wait for ALL of them in front of the value's first use.  The caller waits instead:
+// wait_bias() behind any wait that covers the loads issued up to here (loads return in the order they were issued).
 __device__ inline void load_bias_table(BiasTable &t, const float *rpb_h, int W, int lane) {
-    const Rsrc rs = make_rsrc(rpb_h, rpb_h ? W * 4 : 0);
-    t.raw = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rs, (lane - kBiasPad) * 4, 0, 0));      // outside [0, W): 0
+    const uint64_t p = reinterpret_cast<uint64_t>(rpb_h);
+    const u32x4 rs = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, rpb_h ? (uint32_t)W * 4u : 0u, 0x00020000u};   // NULL: empty, reads as zeros
+    const int off = (lane - kBiasPad) * 4;                                                                         // outside [0, W): 0
+    asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(t.raw) : "v"(off), "s"(rs) : "memory");
 }
-__device__ inline void write_bias_table(LDS_PTR(float) tab, const BiasTable &t, int W, int lane) {
-    tab[lane] = (uint32_t)(lane - kBiasPad) < (uint32_t)W ? t.raw * kLog2e : kNegInf;
+// Ties the value to the wait in front of it, so that nothing that uses it is moved ahead of that wait.
+__device__ inline void wait_bias(BiasTable &t) { asm volatile("" : "+v"(t.raw) :: "memory"); }
+__device__ inline void write_bias_table(LDS_PTR(float) tab, const BiasTable &t, int W, int lane, float mult = kLog2e) {
+    tab[lane] = (uint32_t)(lane - kBiasPad) < (uint32_t)W ? t.raw * mult : kNegInf;
 }
 // The lane's slots out of the wave's own table (written by this wave: program order is enough).
 template <int NBV>
@@ -346,6 +377,15 @@ __device__ inline void read_window(Window<NBV> &w, LDS_PTR(float) tab, int L, in
     }
     w.keep0 = u32x2{m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
     w.keep2 = u32x2{~w.keep0.x, ~w.keep0.y};
+}
+
+// A wave-uniform int32 through the scalar cache: it does not count on the vector-memory counter, so waiting for it
+// does not wait for the strip copies in flight.
+__device__ inline int load_uniform_i32(const int32_t *p, uint32_t index) {
+    const int32_t *a = p + index;
+    int v;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(a) : "memory");
+    return v;
 }
 
 // Kernel arguments live in memory and the compiler fetches each one next to its

@@ -45,8 +45,7 @@ __device__ inline void stage_scores(Rsrc src, int first, LDS_PTR(float) region, 
     for (int j = 0; j < kRounds; ++j) {
         const int c = j * kWaves + wave;
         if (c < chunks)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(src, (LDS_PTR(void))(region + c * (kChunk / 4)), 16,
-                                                     first * 4 + c * kChunk + lane * 16, 0, 0, AUX);
+            load_to_lds<16, AUX>(src, (LDS_PTR(char))(region + c * (kChunk / 4)), first * 4 + c * kChunk + lane * 16);
     }
 }
 

@@ -280,7 +280,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
         const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
         const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch, outl.width);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(ls, (LDS_PTR(void))(lse_lds + 64 * wave), 4, (16 * q0 + tid) * 4, 0, 0, 0);
+        load_to_lds<4, 0>(ls, (LDS_PTR(char))(lse_lds + 64 * wave), (16 * q0 + tid) * 4);
         constexpr int KT = kWideQueryTiles + NBV - 1;
         stage_direct<C, KT, kReadShared>(ks, 16 * q0 - shift, k_lds, ktiles, wave, lane_off, in.pitch);
         stage_direct<C, kWideQueryTiles, kReadShared>(qs, 16 * q0, q_lds, qtiles, wave, lane_off, in.pitch);
