@@ -56,12 +56,9 @@ WORKLOADS = {
 }
 
 
-if os.environ.get("NA1D_BENCH_EXTRA"):      # NAME=N,H,T,C,W,dtype,bwd;... : further shapes for --only
-    for _item in os.environ["NA1D_BENCH_EXTRA"].split(";"):
-        _name, _, _v = _item.partition("=")
-        _f = _v.split(",")
-        WORKLOADS[_name] = dict(N=int(_f[0]), H=int(_f[1]), T=int(_f[2]), C=int(_f[3]), W=int(_f[4]), dtype=_f[5],
-                                bwd=_f[6] == "1", desc="extra shape " + _v)
+def window_left(W):
+    """Slots left of the query in an odd or even window: W - 1 - W // 2 (models/PCF_NATransformer.py:48-49)."""
+    return W - 1 - W // 2
 
 
 def algorithmic_bytes(w):
@@ -211,10 +208,9 @@ def bind_packed(lib, w, sets, with_lse=True):
     """Argument tuples bound once, so that a timed call is one ctypes call."""
     import torch
     from na1d_amd import _lib
-    from oracle import na1d_oracle as O
     H, T, C, W = w["H"], w["T"], w["C"], w["W"]
     B = w["N"] * H
-    _, L = O.split_window(W)
+    L = window_left(W)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     tag = _lib.dtype_tag(sets[0]["q"].dtype)
@@ -235,9 +231,8 @@ def bind_strided(lib, w, sets, with_lse=True, which="both"):
     packed (the same bytes; separates what the reads cost from what the writes cost)."""
     import torch
     from na1d_amd import _lib
-    from oracle import na1d_oracle as O
     N, H, T, C, W = w["N"], w["H"], w["T"], w["C"], w["W"]
-    _, L = O.split_window(W)
+    L = window_left(W)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     tag = _lib.dtype_tag(sets[0]["qkv"].dtype)
@@ -284,10 +279,6 @@ def config_record(lib, clock, name, layout, steps, warmup, device):
     else:
         which = {"strided": "both", "strided_in": "in", "strided_out": "out"}[layout]
         fwd, bwd = bind_strided(lib, w, make_strided_sets(w, n_sets, device), with_lse=w["bwd"], which=which)
-    shift = int(os.environ.get("NA1D_BENCH_BWD_SHIFT", "0"))
-    if bwd and shift:
-        bwd0 = bwd
-        bwd = lambda i: bwd0(i + shift)
     calls = [fwd] + ([bwd] if bwd else [])
     for i in range(max(warmup, n_sets)):
         for f in calls:
@@ -308,11 +299,10 @@ def unfused_record(lib, clock, name, steps, warmup, device):
     4C + 4W algorithmic bytes per token each (16-bit rows in or out, fp32 scores out or in)."""
     import torch
     from na1d_amd import _lib
-    from oracle import na1d_oracle as O
     w = WORKLOADS[name]
     H, T, C, W = w["H"], w["T"], w["C"], w["W"]
     B = w["N"] * H
-    _, L = O.split_window(W)
+    L = window_left(W)
     dt = _dtype(w)
     nbytes = B * T * (4 * C + 4 * W)
     n = max(2, int(ROTATE_BYTES // nbytes) + 1)
@@ -336,6 +326,96 @@ def unfused_record(lib, clock, name, steps, warmup, device):
         (ms, kname), = clock.run([f], steps)
         rec[key] = kernel_record(ms, kname, nbytes)
     del rows, other, outs, attn
+    torch.cuda.empty_cache()
+    return rec
+
+
+MFMA_PEAK_TFLOPS = 2500.0      # dense bf16 / fp16 matrix-core peak of MI355X
+
+# Windows the two/three-block kernels do not cover run the wide kernels: the reference allows up to 80 slots
+# (models/PCF_NATransformer.py:53).  name: (N, H, T, C, W, dtype)
+WIDE_WORKLOADS = {
+    "wide33": dict(N=128, H=8, T=300, C=32, W=33, dtype="fp16", bwd=True,
+                   desc="NA1D fwd+bwd fp16 batch=128 heads=8 T=300 head_dim=32 window=33 (wide-window kernels)"),
+    "wide65": dict(N=128, H=8, T=300, C=32, W=65, dtype="fp16", bwd=True,
+                   desc="NA1D fwd+bwd fp16 batch=128 heads=8 T=300 head_dim=32 window=65 (wide-window kernels)"),
+}
+
+# The two dense (GlobalAttention) layers of each model (models/PCF_NATransformer.py:181-225): 4 heads of 64 channels.
+GLOBAL_WORKLOADS = {
+    "global_cfg3": dict(N=256, H=4, T=100, C=64, dtype="bf16", bwd=False,
+                        desc="dense layer of PCF-NAT 4x4 inference: batch=256 heads=4 T=100 head_dim=64, fwd bf16"),
+    "global_cfg4": dict(N=64, H=4, T=1000, C=64, dtype="bf16", bwd=False,
+                        desc="dense layer of PCF-NAT 6x4 at max length: batch=64 heads=4 T=1000 head_dim=64, fwd bf16"),
+    "global_cfg5": dict(N=128, H=4, T=100, C=64, dtype="fp16", bwd=True,
+                        desc="dense layer of MFA-NAT 4x4 training: batch=128 heads=4 T=100 head_dim=64, fwd+bwd fp16"),
+}
+
+
+def wide_record(lib, clock, name, steps, warmup, device):
+    """Forward and backward kernel of one wide-window shape (packed layout), bytes as for the other fused kernels."""
+    import torch
+    w = WIDE_WORKLOADS[name]
+    n_sets = n_sets_for(w)
+    fwd, bwd = bind_packed(lib, w, make_packed_sets(w, n_sets, device), with_lse=True)
+    for i in range(max(warmup, n_sets)):
+        fwd(i)
+        bwd(i)
+    torch.cuda.synchronize()
+    timed = clock.run([fwd, bwd], steps)
+    fb, bb = algorithmic_bytes(w)
+    rec = {"name": name, "workload": w["desc"], "B": w["N"] * w["H"], "T": w["T"], "C": w["C"], "W": w["W"],
+           "dtype": w["dtype"], "launches": steps, "forward": kernel_record(*timed[0], fb),
+           "backward": kernel_record(*timed[1], bb)}
+    torch.cuda.empty_cache()
+    return rec
+
+
+def global_record(lib, clock, name, steps, warmup, device):
+    """Dense attention at one of the models' shapes.  These kernels are bound by the matrix cores and LDS, not by HBM:
+    the record gives TFLOP/s against the dense 16-bit matrix-core peak, counting 4*T*T*C flop per sequence forward
+    (Q.K^T and P.V) and 10*T*T*C backward (five products of that size), next to the bytes moved."""
+    import torch
+    from na1d_amd import _lib
+    w = GLOBAL_WORKLOADS[name]
+    N, H, T, C = w["N"], w["H"], w["T"], w["C"]
+    B, dt = N * H, _dtype(w)
+    n = max(2, int(ROTATE_BYTES // (B * T * C * 2 * (11 if w["bwd"] else 4))) + 1)
+    g = torch.Generator(device="cpu").manual_seed(0)
+    sets = []
+    for _ in range(n):
+        st = {k_: torch.randn(B, T, C, generator=g).to(dt).to(device) for k_ in ("q", "k", "v", "do")}
+        st["o"], st["lse"] = torch.empty_like(st["q"]), torch.empty(B, T, dtype=torch.float32, device=device)
+        if w["bwd"]:
+            for k_ in ("dq", "dk", "dv"):
+                st[k_] = torch.empty_like(st["q"])
+            st["ws"] = torch.empty(_lib.global_backward_workspace_bytes(B, H, T, C, dt), dtype=torch.uint8, device=device)
+        sets.append(st)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    tag, scale = _lib.dtype_tag(dt), C ** -0.5
+    fa = [(P(s["o"]), P(s["lse"]), P(s["q"]), P(s["k"]), P(s["v"]), None, B, H, T, C, scale, tag, 0.0, 0, stream) for s in sets]
+    fwd = lambda i: _lib.check(lib.na1d_global_forward(*fa[i % n]), "na1d_global_forward")
+    calls = [fwd]
+    if w["bwd"]:
+        ba = [(P(s["dq"]), P(s["dk"]), P(s["dv"]), P(s["q"]), P(s["k"]), P(s["v"]), P(s["o"]), P(s["do"]), P(s["lse"]), None,
+               B, H, T, C, scale, tag, 0.0, 0, P(s["ws"]), s["ws"].numel(), stream) for s in sets]
+        calls.append(lambda i: _lib.check(lib.na1d_global_backward(*ba[i % n]), "na1d_global_backward"))
+    for i in range(max(warmup, n)):
+        for f in calls:
+            f(i)
+    torch.cuda.synchronize()
+    timed = clock.run(calls, steps)
+
+    def rec_of(ms, kname, flop, nbytes):
+        return {"kernel": kname, "kernel_us": round(ms * 1e3, 3), "flop": flop, "TFLOPs": round(flop / (ms * 1e-3) / 1e12, 2),
+                "frac_of_mfma_peak": round(flop / (ms * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, 4), "algorithmic_bytes": nbytes,
+                "GBps": round(nbytes / (ms * 1e-3) / 1e9, 1)}
+
+    rec = {"name": name, "workload": w["desc"], "B": B, "T": T, "C": C, "dtype": w["dtype"], "launches": steps,
+           "forward": rec_of(*timed[0], 4 * T * T * C * B, 8 * C * B * T),
+           "backward": rec_of(*timed[1], 10 * T * T * C * B, (18 * C + 8) * B * T) if w["bwd"] else None}
+    del sets
     torch.cuda.empty_cache()
     return rec
 
@@ -533,7 +613,6 @@ def main():
 
     import torch
     from na1d_amd import _lib
-    from oracle import na1d_oracle as O
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     lib = _lib.load()
@@ -546,7 +625,11 @@ def main():
     if args.only:
         name, _, layout = args.only.partition(":")
         layout = layout or "packed"
-        if layout == "unfused":
+        if name in WIDE_WORKLOADS:
+            print(json.dumps(wide_record(lib, clock, name, args.steps, args.warmup, dev)))
+        elif name in GLOBAL_WORKLOADS:
+            print(json.dumps(global_record(lib, clock, name, args.steps, args.warmup, dev)))
+        elif layout == "unfused":
             print(json.dumps(unfused_record(lib, clock, name, args.steps, args.warmup, dev)))
         else:
             print(json.dumps(config_record(lib, clock, name, layout, args.steps, args.warmup, dev)))
@@ -555,7 +638,7 @@ def main():
     w = WORKLOADS[args.workload]
     H, T, C, W = w["H"], w["T"], w["C"], w["W"]
     B = w["N"] * H
-    _, L = O.split_window(W)
+    L = window_left(W)
     fwd_bytes, bwd_bytes = algorithmic_bytes(w)
     set_bytes = fwd_bytes + bwd_bytes
     n_sets = n_sets_for(w)
@@ -622,17 +705,23 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_configs:
         per_cfg = max(50, min(K, 100))          # launches per kernel and configuration
-        recs, unf = [], []
+        recs, unf, wide, dense = [], [], [], []
         try:
             for name in sorted(WORKLOADS):
                 for layout in ("packed", "strided"):
                     recs.append(config_record(lib, clock, name, layout, per_cfg, 10, dev))
             for name in ("cfg2", "cfg3"):
                 unf.append(unfused_record(lib, clock, name, per_cfg, 10, dev))
+            for name in sorted(WIDE_WORKLOADS):
+                wide.append(wide_record(lib, clock, name, per_cfg, 10, dev))
+            for name in sorted(GLOBAL_WORKLOADS):
+                dense.append(global_record(lib, clock, name, per_cfg, 10, dev))
         except Exception as e:      # extra records must not take the headline line down with them
             recs.append({"error": "%s: %s" % (type(e).__name__, str(e)[:300])})
         line["configs"] = recs
         line["unfused"] = unf
+        line["wide"] = wide
+        line["global"] = dense
         shapes = {}
         for name, cw in sorted(WORKLOADS.items()):
             one = cw["N"] * cw["H"] * cw["T"] * cw["C"] * 2

@@ -45,6 +45,8 @@ extern "C" {
 #define NA1D_ERR_LAUNCH      -7   /* the HIP runtime rejected the launch              */
 #define NA1D_ERR_UNSUPPORTED -8   /* valid arguments that no built kernel covers      */
 #define NA1D_ERR_TOO_LARGE   -9   /* the problem needs more than the static scratch   */
+#define NA1D_ERR_WORKSPACE   -10  /* a workspace was passed that is too small         */
+#define NA1D_ERR_SCALE       -11  /* scale is not a finite number above zero          */
 
 #define NA1D_MAX_WINDOW 80
 
@@ -101,7 +103,8 @@ int na1d_v_backward(void *dv, const void *attn, const void *dout,
  *              A slot gets the additive -100 of the reference when its query
  *              row t >= t_valid or its key lies outside [0, t_valid).
  *   scale    : multiplies the fp32 scores (pass 1.0f when q is pre-scaled, as
- *              the reference model does)
+ *              the reference model does); finite and > 0 (the reference's is
+ *              head_dim^-0.5), otherwise NA1D_ERR_SCALE
  *   lse      : fp32 [B, T] out, log-sum-exp of each row's logits (for backward);
  *              may be NULL for inference
  */
@@ -121,8 +124,9 @@ int na1d_fused_forward(void *out, float *lse,
  *   workspace, workspace_bytes : optional device scratch for the d rpb reduction.
  *          With at least na1d_fused_backward_workspace_bytes(...) bytes the per-
  *          workgroup partial sums go there and a second small kernel folds them in a
- *          fixed order; with NULL / too few bytes they are added with float atomics
- *          (slower under contention, order not reproducible).  Contents need no
+ *          fixed order; with NULL they are added with float atomics (slower under
+ *          contention, order not reproducible).  A non-NULL workspace of too few bytes
+ *          is refused with NA1D_ERR_WORKSPACE rather than ignored.  Contents need no
  *          initialisation and are not meaningful afterwards.
  */
 int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb,
@@ -227,7 +231,7 @@ int na1d_fused_backward_strided_dropout(void *dq, void *dk, void *dv, float *drp
  * lse [B, T] fp32 (natural log; may be NULL in the forward when no backward follows).  The probabilities are never
  * written to memory.  The backward needs a workspace of na1d_global_backward_workspace_bytes() bytes (one fp32 per
  * row: rowsum(dout * out)) and writes every gradient exactly once, so it is deterministic.
- * C % 8 == 0; C > 128 returns NA1D_ERR_UNSUPPORTED.  p_drop, seed: attention dropout (attn_drop of
+ * C % 8 == 0; C > 128 returns NA1D_ERR_UNSUPPORTED.  scale: finite and > 0 as in na1d_fused_forward.  p_drop, seed: attention dropout (attn_drop of
  * models/PCF_NATransformer.py:193,218; 0 in the reference's configurations) by the keep rule stated at
  * na1d_fused_forward_dropout with the key's row index as the slot j; 0 <= p_drop < 1, 0 switches it off.
  */
@@ -286,7 +290,10 @@ int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int
  * NA1D_NOALLOC_SCRATCH_BYTES (32768 workgroups), otherwise NA1D_ERR_TOO_LARGE.  All calls on one GPU share that
  * GPU's array: calls that overlap in time on one GPU (different streams or threads) race on it; calls on one
  * stream are ordered and safe.  The array needs no clearing between calls: a call writes every entry it reads.
- * The device that owns `stream` must be the current device.
+ * The device that owns `stream` must be the current device.  The first call on a device looks the array's address
+ * up (hipGetSymbolAddress): make that call outside stream capture; later ones record nothing but their two kernels.
+ * While na1d_force_generic(1) is on the call returns NA1D_ERR_UNSUPPORTED like the strided entry points (the generic
+ * kernels have no fixed-order reduction).
  */
 #define NA1D_NOALLOC_SCRATCH_BYTES (4 * 1024 * 1024)
 int na1d_fused_backward_noalloc(void *dq, void *dk, void *dv, float *drpb,

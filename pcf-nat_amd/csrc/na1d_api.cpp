@@ -18,6 +18,8 @@ namespace {
 using na1d::Geom;
 
 inline bool misaligned(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+// The kernels fold the bias into the scores before the scale, which takes a positive one (false for NaN too).
+inline bool bad_scale(float scale) { return !(scale > 0.f && scale <= 3.0e38f); }
 
 // Shape checks shared by every entry point.  Returns NA1D_OK, an error, or +1 for
 // "nothing to do".
@@ -129,6 +131,8 @@ const char *na1d_status_string(int status) {
         case NA1D_ERR_LAUNCH: return "HIP rejected the kernel launch";
         case NA1D_ERR_UNSUPPORTED: return "no kernel built for these arguments";
         case NA1D_ERR_TOO_LARGE: return "the problem needs more scratch than NA1D_NOALLOC_SCRATCH_BYTES";
+        case NA1D_ERR_WORKSPACE: return "the workspace is smaller than the size the *_workspace_bytes() query returns";
+        case NA1D_ERR_SCALE: return "scale must be a finite number above zero";
         default: return "unknown status";
     }
 }
@@ -173,6 +177,7 @@ int na1d_fused_forward(void *out, float *lse, const void *q, const void *k, cons
                        const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
                        int64_t left, float scale, int dtype, void *stream) {
     NA1D_CHECK(out, q, k, B, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
     const na1d::Layout packed = na1d::packed_layout(g);
@@ -189,6 +194,7 @@ int na1d_fused_backward(void *dq, void *dk, void *dv, float *drpb, const void *q
                         int64_t left, float scale, int dtype, void *workspace, int64_t workspace_bytes,
                         void *stream) {
     NA1D_CHECK(dq, q, k, B, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
         return NA1D_ERR_ALIGN;
@@ -209,6 +215,7 @@ int na1d_fused_forward_strided(void *out, float *lse, const void *q, const void 
                                const int64_t *out_strides, void *stream) {
     if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
     NA1D_CHECK(out, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
     na1d::Layout in, outl;
@@ -226,6 +233,7 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb, const
                                 void *stream) {
     if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
     NA1D_CHECK(dq, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!dk || !dv || !v || !dout || !lse) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(dout)) return NA1D_ERR_ALIGN;
     if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
@@ -241,6 +249,7 @@ int na1d_fused_forward_dropout(void *out, float *lse, const void *q, const void 
                                const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
                                int64_t left, float scale, int dtype, float p_drop, uint64_t seed, void *stream) {
     NA1D_CHECK(out, q, k, B, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
     if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
@@ -259,6 +268,7 @@ int na1d_fused_backward_dropout(void *dq, void *dk, void *dv, float *drpb, const
                                 int64_t left, float scale, int dtype, float p_drop, uint64_t seed, void *workspace,
                                 int64_t workspace_bytes, void *stream) {
     NA1D_CHECK(dq, q, k, B, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
         return NA1D_ERR_ALIGN;
@@ -283,6 +293,7 @@ int na1d_fused_forward_strided_dropout(void *out, float *lse, const void *q, con
                                        void *stream) {
     if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
     NA1D_CHECK(out, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
     if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
@@ -306,6 +317,7 @@ int na1d_fused_backward_strided_dropout(void *dq, void *dk, void *dv, float *drp
                                         void *stream) {
     if (N < 0 || H < 1 || N > INT64_MAX / H) return NA1D_ERR_SHAPE;
     NA1D_CHECK(dq, q, k, N * H, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!dk || !dv || !v || !dout || !lse) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(dout)) return NA1D_ERR_ALIGN;
     if (workspace && misaligned(workspace)) return NA1D_ERR_ALIGN;
@@ -326,6 +338,7 @@ int na1d_global_forward(void *out, float *lse, const void *q, const void *k, con
                         int64_t B, int64_t H, int64_t T, int64_t C, float scale, int dtype, float p_drop, uint64_t seed,
                         void *stream) {
     NA1D_CHECK(out, q, k, B, T, C, 1, 0, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!v) return NA1D_ERR_NULL;
     if (misaligned(v)) return NA1D_ERR_ALIGN;
     if (!(p_drop >= 0.f && p_drop < 1.f)) return NA1D_ERR_SHAPE;
@@ -338,6 +351,7 @@ int na1d_global_backward(void *dq, void *dk, void *dv, const void *q, const void
                          int64_t C, float scale, int dtype, float p_drop, uint64_t seed, void *workspace,
                          int64_t workspace_bytes, void *stream) {
     NA1D_CHECK(dq, q, k, B, T, C, 1, 0, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!dk || !dv || !v || !out || !dout || !lse || !workspace) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout) || misaligned(workspace))
         return NA1D_ERR_ALIGN;
@@ -353,9 +367,11 @@ int na1d_fused_backward_noalloc(void *dq, void *dk, void *dv, float *drpb, const
                                 const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
                                 int64_t left, float scale, int dtype, void *stream) {
     NA1D_CHECK(dq, q, k, B, T, C, W, left, H, dtype, g);
+    if (bad_scale(scale)) return NA1D_ERR_SCALE;
     if (!dk || !dv || !v || !out || !dout || !lse) return NA1D_ERR_NULL;
     if (misaligned(dk) || misaligned(dv) || misaligned(v) || misaligned(out) || misaligned(dout))
         return NA1D_ERR_ALIGN;
+    if (!mfma_allowed()) return NA1D_ERR_UNSUPPORTED;      // the generic kernels have no fixed-order reduction
     const int64_t need = na1d::mfma::fused_bwd_workspace_bytes(g, dtype);
     if (need <= 0) return NA1D_ERR_UNSUPPORTED;
     if (need > na1d::mfma::kStaticScratchBytes) return NA1D_ERR_TOO_LARGE;

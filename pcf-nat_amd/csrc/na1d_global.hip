@@ -420,8 +420,9 @@ int launch_global_fwd(void *out, float *lse, const void *q, const void *k, const
     a.scale = scale;
     auto kern = g.drop.threshold ? global_fwd_kernel<DT, C, true> : global_fwd_kernel<DT, C, false>;
     if (!allow_lds(kern, global_lds<C>(3))) return NA1D_ERR_LAUNCH;
-    kern<<<(unsigned)items, kThreads, global_lds<C>(3), s>>>((char *)out, lse, (const char *)q, (const char *)k,
-                                                            (const char *)v, t_valid, (uint32_t)items, a);
+    note_kernel_as("global_fwd_kernel<%s, %d, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C, g.drop.threshold ? "true" : "false");
+    launch_kernel(kern, (unsigned)items, global_lds<C>(3), s, (char *)out, lse, (const char *)q, (const char *)k,
+                  (const char *)v, t_valid, (uint32_t)items, a);
     return launch_status();
 }
 
@@ -436,12 +437,14 @@ int launch_global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q,
     auto dq_kern = g.drop.threshold ? global_dq_kernel<DT, C, true> : global_dq_kernel<DT, C, false>;
     auto dkv_kern = g.drop.threshold ? global_dkv_kernel<DT, C, true> : global_dkv_kernel<DT, C, false>;
     if (!allow_lds(dq_kern, global_lds<C>(5)) || !allow_lds(dkv_kern, global_lds<C>(4))) return NA1D_ERR_LAUNCH;
-    dq_kern<<<(unsigned)items, kThreads, global_lds<C>(5), s>>>((char *)dq, delta, (const char *)q, (const char *)k,
-                                                               (const char *)v, (const char *)out, (const char *)dout, lse,
-                                                               t_valid, (uint32_t)items, a);
-    dkv_kern<<<(unsigned)items, kThreads, global_lds<C>(4), s>>>((char *)dk, (char *)dv, (const char *)q, (const char *)k,
-                                                                (const char *)v, (const char *)dout, lse, delta, t_valid,
-                                                                (uint32_t)items, a);
+    // the pair of profiling events, if set, spans both kernels
+    note_kernel_as("global_dq_kernel + global_dkv_kernel<%s, %d, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C,
+                   g.drop.threshold ? "true" : "false");
+    launch_kernel_span(1, dq_kern, (unsigned)items, (unsigned)kThreads, global_lds<C>(5), s, (char *)dq, delta, (const char *)q,
+                       (const char *)k, (const char *)v, (const char *)out, (const char *)dout, lse, t_valid, (uint32_t)items, a);
+    launch_kernel_span(2, dkv_kern, (unsigned)items, (unsigned)kThreads, global_lds<C>(4), s, (char *)dk, (char *)dv,
+                       (const char *)q, (const char *)k, (const char *)v, (const char *)dout, lse, delta, t_valid,
+                       (uint32_t)items, a);
     return launch_status();
 }
 

@@ -10,14 +10,8 @@ namespace mfma {
 // =============================================================================
 // Fused forward
 // =============================================================================
-#ifndef NA1D_HG_MT
-#define NA1D_HG_MT 4
-#endif
-constexpr int kGroupTiles = NA1D_HG_MT;      // tiles per strip when heads are staged in groups
-#ifndef NA1D_HG_WAVES
-#define NA1D_HG_WAVES 8
-#endif
-constexpr int kGroupWaves = NA1D_HG_WAVES;   // waves per workgroup when heads are staged in groups: a group's regions are
+constexpr int kGroupTiles = 4;               // tiles per strip when heads are staged in groups
+constexpr int kGroupWaves = 8;               // waves per workgroup when heads are staged in groups: a group's regions are
                                              // 2-4 times a head's, and twice the waves keep as many tiles in flight per CU
 
 // HG heads whose rows lie side by side in memory (a projection's output, head h of a token right behind head h-1)
@@ -351,9 +345,7 @@ drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, 
 
 // Waves per SIMD the register allocation of the backward must leave room for.  16-channel heads: the LDS footprint
 // admits six workgroups per CU, so the registers must too (80 or fewer; the dropout variant would spill and is left alone).
-#ifndef NA1D_BWD_MIN_WAVES
-#define NA1D_BWD_MIN_WAVES(C, DROP) ((C) == 16 && !(DROP) ? 6 : 1)
-#endif
+constexpr int bwd_min_waves(int C, bool drop) { return C == 16 && !drop ? 6 : 1; }
 
 // Rows that no other workgroup reads: the backward takes them with the workgroup-scope policy rather than the
 // non-temporal one of the forward (measured: 4-7 % on the 16-channel backward, nothing either way at 32 channels; the
@@ -361,15 +353,11 @@ drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, 
 constexpr int kReadOnceBwd = 1;
 constexpr int kBwdMinItems = 256;      // fewer items than this: shorter strips
 template <int C> struct StripBwd {
-#ifdef NA1D_BWD_MT
-    static constexpr int kMaxTiles = NA1D_BWD_MT * 32 / (C < 32 ? 32 : C);
-#else
     static constexpr int kMaxTiles = C <= 32 ? 8 : C <= 64 ? 4 : 2;
-#endif
 };
 
 template <class DT, int C, int NBV, bool DROP>
-__global__ void __launch_bounds__(kThreads, NA1D_BWD_MIN_WAVES(C, DROP))
+__global__ void __launch_bounds__(kThreads, bwd_min_waves(C, DROP))
 fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, float *__restrict__ drpb,
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
@@ -708,8 +696,13 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                hipStream_t s) {
     const Split sp = make_split(g.B, g.T, StripBwd<C>::kMaxTiles, kBwdMinItems);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
+    // a workspace that is passed is used or refused: falling back to atomics would silently give up the fixed order
+    // the caller asked for
     float *partial = nullptr;
-    if (drpb && workspace && workspace_bytes >= sp.items * kPartialStride * (int64_t)sizeof(float)) partial = workspace;
+    if (drpb && workspace) {
+        if (workspace_bytes < sp.items * kPartialStride * (int64_t)sizeof(float)) return NA1D_ERR_WORKSPACE;
+        partial = workspace;
+    }
     const bool two = window_blocks(g) == 2;
     auto kern = g.drop.threshold ? (two ? fused_bwd_kernel<DT, C, 2, true> : fused_bwd_kernel<DT, C, 3, true>)
                                  : (two ? fused_bwd_kernel<DT, C, 2, false> : fused_bwd_kernel<DT, C, 3, false>);
@@ -724,7 +717,8 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
                   div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g), g.drop);
-    if (partial && drpb)
+    // not behind a launch that was refused (events set on a capturing stream): the sums it would fold do not exist
+    if (partial && drpb && !launch_events().refused)
         drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();
 }

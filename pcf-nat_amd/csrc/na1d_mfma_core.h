@@ -60,10 +60,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 #define LDS_PTR(T) __attribute__((address_space(3))) T *
 
-#ifndef NA1D_WAVES
-#define NA1D_WAVES 4
-#endif
-constexpr int kWaves = NA1D_WAVES;   // waves per workgroup
+constexpr int kWaves = 4;            // waves per workgroup
 constexpr int kThreads = 64 * kWaves;
 constexpr float kNegInf = -__builtin_inff();
 
@@ -134,11 +131,7 @@ template <int C> struct Lds {
 
 // Tiles per strip (compile-time ceiling that sizes LDS and the copy loops).
 template <int C> struct Strip {
-#ifdef NA1D_FWD_MT
-    static constexpr int kMaxTiles = NA1D_FWD_MT * 32 / (C < 32 ? 32 : C);
-#else
-    static constexpr int kMaxTiles = C <= 16 ? 8 : C <= 32 ? 8 : C <= 64 ? 4 : 2;
-#endif
+    static constexpr int kMaxTiles = C <= 32 ? 8 : C <= 64 ? 4 : 2;
 };
 
 // Copy up to NTILES tiles of rows, starting at row_lo of a sequence, into an LDS
@@ -481,21 +474,34 @@ inline void note_kernel(const char *base, int dtype, int C, int nbv, int drop = 
         snprintf(ev.kernel, sizeof ev.kernel, "%s<%s, %d, %d, %s, %d>", base, dt, C, nbv, drop ? "true" : "false", hg);
 }
 
-// Launch, with the calling thread's profiling events around the kernel if it has set any.
+// The same for kernels with other template arguments: the name is spelt out by the caller.
+template <class... A> inline void note_kernel_as(const char *format, A... a) {
+    LaunchEvents &ev = launch_events();
+    if (ev.start || ev.stop) snprintf(ev.kernel, sizeof ev.kernel, format, a...);
+}
+
+// Launch, with the calling thread's profiling events around the kernel if it has set any.  An operator of several
+// kernels gives the first one the start event and the last one the stop event (`span`: bit 0 = this launch records
+// start, bit 1 = it records stop).
 template <class K, class... Args>
-inline void launch_kernel_block(K kern, unsigned grid, unsigned block, size_t lds, hipStream_t s, Args... args) {
+inline void launch_kernel_span(int span, K kern, unsigned grid, unsigned block, size_t lds, hipStream_t s, Args... args) {
     LaunchEvents &ev = launch_events();
     if (ev.start || ev.stop) {
         // events recorded by the launch itself do not belong in a captured graph: refuse instead of recording them
         hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
-            ev.refused = true;
+        if (ev.refused || hipStreamIsCapturing(s, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+            ev.refused = true;      // also what follows a refused launch in the same call
             return;
         }
-        hipExtLaunchKernelGGL(kern, dim3(grid), dim3(block), (uint32_t)lds, s, ev.start, ev.stop, 0, args...);
+        hipExtLaunchKernelGGL(kern, dim3(grid), dim3(block), (uint32_t)lds, s, (span & 1) ? ev.start : nullptr,
+                              (span & 2) ? ev.stop : nullptr, 0, args...);
     } else {
         kern<<<grid, block, lds, s>>>(args...);
     }
+}
+template <class K, class... Args>
+inline void launch_kernel_block(K kern, unsigned grid, unsigned block, size_t lds, hipStream_t s, Args... args) {
+    launch_kernel_span(3, kern, grid, block, lds, s, args...);
 }
 template <class K, class... Args>
 inline void launch_kernel(K kern, unsigned grid, size_t lds, hipStream_t s, Args... args) {

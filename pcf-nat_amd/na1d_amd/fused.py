@@ -54,11 +54,21 @@ def _strided_or_packed_backward(dq4, dk4, dv4, drpb, q4, k4, v4, packed_out, dou
         dst.copy_(src.view(N, H, T, C))
 
 
-def _deterministic_workspace(B, H, T, C, win_size, left, like):
+def _deterministic_workspace_bytes(B, H, T, C, win_size, left, dilation, dtype):
+    """Bytes of scratch for the fixed-order reduction of the bias gradient over every launch of one backward: with
+    dilation d the residue classes have ceil(T/d) or floor(T/d) rows, and the shorter class can need the larger
+    workspace (the split into workgroups is not monotonic in the length), so it is the maximum over both."""
+    lengths = {-(-T // dilation)}
+    if dilation > 1 and T % dilation and T // dilation > 0:
+        lengths.add(T // dilation)
+    return max(_lib.fused_backward_workspace_bytes(B, H, t, C, win_size, left, dtype) for t in lengths)
+
+
+def _deterministic_workspace(B, H, T, C, win_size, left, like, dilation=1):
     """Scratch for the fixed-order reduction of the bias gradient.  Only the two/three-block matrix-core backward
     has that path; for the shapes it does not cover (wide windows, head_dim > 128) the library would fall back to
     float atomics silently, so the request is refused instead."""
-    nbytes = _lib.fused_backward_workspace_bytes(B, H, T, C, win_size, left, like.dtype)
+    nbytes = _deterministic_workspace_bytes(B, H, T, C, win_size, left, dilation, like.dtype)
     if nbytes <= 0:
         raise _lib.NA1DError("deterministic=True: no fixed-order reduction of the bias gradient for head_dim %d, "
                              "window %d (left %d); it covers head_dim <= 128 and windows of at most 32 slots with "
@@ -116,7 +126,7 @@ class _FusedNA1D(torch.autograd.Function):
         if rpb is not None and ctx.needs_input_grad[3]:
             drpb = torch.zeros((num_heads, win_size), dtype=torch.float32, device=q.device)
             if deterministic:   # fold the per-workgroup partial sums in a fixed order instead of with atomics
-                ws = _deterministic_workspace(B, num_heads, -(-T // dilation), C, win_size, left, q)
+                ws = _deterministic_workspace(B, num_heads, T, C, win_size, left, q, dilation)
         if dilation == 1:
             _lib.call_fused_backward(dq, dk, dv, drpb, q, k, v, out, dout, lses[0], rpb, t_valid,
                                      B, num_heads, T, C, win_size, left, scale, workspace=ws, dropout=ctx.dropout)
@@ -220,7 +230,7 @@ class _FusedNA1DQKV(torch.autograd.Function):
         if rpb is not None and ctx.needs_input_grad[1]:
             drpb = torch.zeros((H, win_size), dtype=torch.float32, device=qkv.device)
             if deterministic:
-                ws = _deterministic_workspace(N * H, H, -(-T // dilation), C, win_size, left, qkv)
+                ws = _deterministic_workspace(N * H, H, T, C, win_size, left, qkv, dilation)
         views = [dqkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)] + [qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)]
         for r, lse in enumerate(lses):
             a = [_residue(z, r, dilation) for z in views]

@@ -402,6 +402,9 @@ class NAttention(nn.Module):
         t = x.shape[-1] if self.channels_first else x.shape[1]
         h, w, left = self.num_heads, self.win_size, self.left
         if self.training:       # the reference trains with its constructor-time mask: fixed length, nothing padded (PCF :131-132)
+            # that mask has `frames` rows, so any other length fails there (a shape error in the addition); it fails here too
+            assert t == self.attn_mask.shape[-2], \
+                "training uses the fixed-length mask built for %d tokens, got %d" % (self.attn_mask.shape[-2], t)
             padding = None
         t_valid = None if padding is None else (t - padding).to(torch.int32)
         dropping = self.attn_drop > 0.0 and self.training

@@ -31,8 +31,8 @@ def test_library_exports_every_declared_symbol():
 def test_status_strings():
     lib = _lib.load()
     assert lib.na1d_status_string(0) == b"ok"
-    for code in range(-9, 0):
-        assert len(lib.na1d_status_string(code)) > 3
+    for code in range(-11, 0):
+        assert len(lib.na1d_status_string(code)) > 3 and lib.na1d_status_string(code) != b"unknown status"
     assert lib.na1d_status_string(-99) == b"unknown status"
 
 
@@ -79,11 +79,51 @@ def test_fused_entry_points_validate():
     assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, None, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, None, 0, None) == -1  # lse
     assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 90, 2, 1.0, 0, None, 0, None) == -4
     assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, P(0x1008), 64, None) == -6
+    # scale has to be a finite number above zero (the reference's is head_dim ** -0.5)
+    for bad in (0.0, -0.25, float("nan"), float("inf")):
+        assert f(ok, None, ok, ok, ok, None, None, 4, 2, 8, 16, 5, 2, bad, 0, None) == -11
+        assert b(ok, ok, ok, None, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 5, 2, bad, 0, None, 0, None) == -11
+    # a workspace that is passed but too small is refused before anything is launched (d rpb asked for)
+    assert b(ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, None, None, 4, 2, 8, 16, 5, 2, 1.0, 0, ok, 64, None) == -10
     w = lib.na1d_fused_backward_workspace_bytes
     assert w(4096, 16, 100, 16, 27, 13, 0) == 4096 * 32 * 4      # one 32-float row per work item
     assert w(1024, 8, 300, 32, 15, 7, 1) > 0
     assert w(4, 2, 8, 136, 5, 2, 0) == 0                         # generic kernel: no workspace
     assert w(4, 3, 8, 16, 5, 2, 0) == -5 and w(4, 2, 8, 16, 99, 2, 0) == -4
+
+
+def test_noalloc_entry_point_validates_and_respects_the_kernel_family_switch():
+    """na1d_fused_backward_noalloc checks its arguments like na1d_fused_backward and, while the generic kernels are
+    forced, reports that it has no kernel (they have no fixed-order reduction)."""
+    lib = _lib.load()
+    ok = ctypes.c_void_p(0x1000)
+    f = lib.na1d_fused_backward_noalloc
+    args = lambda **kw: [ok, ok, ok, None, ok, ok, ok, ok, ok, kw.get("lse", ok), None, None, kw.get("B", 4), 2, 8,
+                         kw.get("C", 16), kw.get("W", 5), 2, kw.get("scale", 1.0), 0, None]
+    assert f(*args(lse=None)) == -1 and f(*args(C=20)) == -3 and f(*args(W=99)) == -4 and f(*args(scale=0.0)) == -11
+    assert f(*args(B=0)) == 0                        # nothing to do
+    assert f(*args(C=136)) == -8 and f(*args(W=40)) == -8        # shapes without a fixed-order reduction
+    assert f(*args(B=1 << 20)) == -9                 # more workgroups than the static scratch holds rows for
+    was = lib.na1d_force_generic(1)
+    try:
+        assert f(*args()) == -8
+    finally:
+        lib.na1d_force_generic(was)
+
+
+def test_deterministic_workspace_covers_every_residue_class():
+    """With dilation d the backward runs once per residue class t mod d, on ceil(T/d) or floor(T/d) rows, all with one
+    workspace.  The split into workgroups is not monotonic in the length (64 sequences: 129 rows need 24576 bytes,
+    128 rows 32768), so the workspace has to be sized over every class, not for the longest."""
+    from na1d_amd import fused
+    w = lambda B, T: _lib.fused_backward_workspace_bytes(B, 4, T, 16, 27, 13, torch.bfloat16)
+    assert w(64, 129) < w(64, 128)                   # the case in point
+    assert fused._deterministic_workspace_bytes(64, 4, 257, 16, 27, 13, 2, torch.bfloat16) == w(64, 128)
+    for B in (4, 64, 256, 4096):
+        for T in (1, 2, 3, 31, 100, 129, 257, 300, 1000):
+            for d in (1, 2, 3, 4, 7):
+                need = max(w(B, -(-(T - r) // d)) for r in range(min(d, T)))
+                assert fused._deterministic_workspace_bytes(B, 4, T, 16, 27, 13, d, torch.bfloat16) == need, (B, T, d)
 
 
 def test_strided_entry_points_validate():

@@ -272,6 +272,52 @@ def test_strided_entry_points_leave_the_gaps_alone(dtype):
     assert not torch.isnan(gbuf[..., :C]).any()
 
 
+@pytest.mark.parametrize("geom", [(2, 16, 100, 16, 27, 13, 24), (3, 8, 75, 32, 15, 7, 40), (2, 4, 37, 16, 27, 13, 8),
+                                  (1, 2, 21, 32, 17, 8, 0)], ids=lambda g: "x".join(map(str, g)))
+@pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
+def test_grouped_heads_keep_to_their_rows(geom, dtype):
+    """Projection layout with head groups (four heads of 16 channels or two of 32 staged together, output rows written
+    back as whole lines out of LDS): T is not a multiple of the tile or the strip, rows are wider than H*C by `gap`
+    sentinel columns, and everything sits between sentinel bands.  Outputs and gradients must be bit-identical to the
+    packed operator and no sentinel may change."""
+    N, H, T, C, W, L, gap = geom
+    g = torch.Generator().manual_seed(11)
+    row = 3 * H * C + gap                                               # elements from one token to the next
+    buf, qkv, pad = _guarded((N, T, row), dtype, 5.0)
+    qkv.copy_(torch.randn(N, T, row, generator=g).to(dtype))
+    qkv[..., 3 * H * C:] = 5.0                                          # the gap columns
+    views = [qkv[..., i * H * C:(i + 1) * H * C].view(N, T, H, C).permute(0, 2, 1, 3) for i in range(3)]
+    orow = H * C + gap
+    obuf, o3, opad = _guarded((N, T, orow), dtype, 5.0)
+    out = o3[..., :H * C].view(N, T, H, C).permute(0, 2, 1, 3)
+    rpb = (torch.randn(H, W, generator=g) * 0.3).cuda()
+    tv = torch.tensor(([T, T // 2, 1] * N)[:N], dtype=torch.int32, device="cuda")
+    lse = torch.empty(N * H, T, device="cuda")
+    assert _lib.call_fused_forward_strided(out, lse, *views, rpb, tv, W, L, 0.5) == 0
+    torch.cuda.synchronize()
+    assert (obuf[:opad] == 5.0).all() and (obuf[opad + o3.numel():] == 5.0).all() and (o3[..., H * C:] == 5.0).all()
+    packed = [z.contiguous().view(N * H, T, C) for z in views]
+    want, want_lse = na1d_fused_forward_lse(*packed, W, L, rpb=rpb, t_valid=tv, num_heads=H, scale=0.5)
+    assert torch.equal(out.contiguous().view(N * H, T, C), want) and torch.equal(lse, want_lse)
+
+    gbuf, gqkv, gpad = _guarded((N, T, row), dtype, 5.0)
+    gviews = [gqkv[..., i * H * C:(i + 1) * H * C].view(N, T, H, C).permute(0, 2, 1, 3) for i in range(3)]
+    dbuf, d3, dpad = _guarded((N, T, orow), dtype, 5.0)
+    d3[..., :H * C] = torch.randn(N, T, H * C, generator=g).to(dtype).cuda()
+    do = d3[..., :H * C].view(N, T, H, C).permute(0, 2, 1, 3)
+    drpb = torch.zeros(H, W, device="cuda")
+    assert _lib.call_fused_backward_strided(*gviews, drpb, *views, do, lse, rpb, tv, W, L, 0.5) == 0
+    torch.cuda.synchronize()
+    assert (gbuf[:gpad] == 5.0).all() and (gbuf[gpad + gqkv.numel():] == 5.0).all() and (gqkv[..., 3 * H * C:] == 5.0).all()
+    wq, wk, wv = (torch.empty_like(want) for _ in range(3))
+    wr = torch.zeros(H, W, device="cuda")
+    _lib.call_fused_backward(wq, wk, wv, wr, *packed, want, do.contiguous().view(N * H, T, C), want_lse, rpb, tv, N * H, H, T, C,
+                             W, L, 0.5)
+    for name, a, b in zip(("dq", "dk", "dv"), gviews, (wq, wk, wv)):
+        assert torch.equal(a.contiguous().view(N * H, T, C), b), name
+    assert torch.allclose(drpb, wr, rtol=1e-4, atol=1e-4)
+
+
 WIDE_GEOMS = [  # (N, H, T, C, W, left): windows the two/three-block kernels do not cover
     (2, 2, 100, 16, 33, 16), (2, 2, 130, 32, 40, 7), (1, 2, 90, 64, 48, 47), (2, 1, 200, 16, 64, 0), (1, 2, 70, 128, 65, 32),
     (2, 2, 300, 32, 80, 39), (1, 3, 45, 16, 80, 79), (2, 2, 17, 32, 80, 0), (1, 1, 500, 64, 27, 20), (2, 2, 64, 16, 31, 30),
@@ -434,6 +480,33 @@ def test_deterministic_rpb_gradient_is_bit_reproducible(C, W, L):
     assert torch.allclose(grads[0][0], grads[2][0], rtol=1e-4, atol=1e-4)
 
 
+def test_deterministic_rpb_gradient_with_dilated_windows():
+    """Dilation 2 on 257 rows: residue classes of 129 and 128 rows, and the 128-row class needs the larger workspace.
+    One workspace sized over both keeps the fixed order for every class: two runs give the same bits."""
+    N, H, T, C, W, L, d = 16, 4, 257, 16, 27, 13, 2
+    q, k, v, do = make_inputs(N * H, T, C, W, 73, torch.float16, n=4, scale=0.25)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(6)) * 0.3
+    assert _lib.fused_backward_workspace_bytes(N * H, H, 129, C, W, L, torch.float16) < \
+        _lib.fused_backward_workspace_bytes(N * H, H, 128, C, W, L, torch.float16)
+    grads = []
+    for det in (True, True, False):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        rd = rpb.cuda().requires_grad_(True)
+        na1d_fused(qd, kd, vd, W, L, rpb=rd, num_heads=H, deterministic=det, dilation=d).backward(do.cuda())
+        grads.append((rd.grad.clone(), qd.grad.clone(), kd.grad.clone(), vd.grad.clone()))
+    assert all(torch.equal(a, b) for a, b in zip(grads[0], grads[1]))
+    assert torch.allclose(grads[0][0], grads[2][0], rtol=1e-4, atol=1e-4)
+    # and the library refuses a workspace that is too small instead of falling back to atomics
+    B = N * H
+    qd, kd, vd, dd = dev(q[:, :128].contiguous(), k[:, :128].contiguous(), v[:, :128].contiguous(), do[:, :128].contiguous())
+    out, lse = torch.empty_like(qd), torch.empty(B, 128, device="cuda")
+    _lib.call_fused_forward(out, lse, qd, kd, vd, rpb.cuda(), None, B, H, 128, C, W, L, 1.0)
+    small = torch.empty(_lib.fused_backward_workspace_bytes(B, H, 129, C, W, L, torch.float16), dtype=torch.uint8, device="cuda")
+    with pytest.raises(_lib.NA1DError, match="workspace"):
+        _lib.call_fused_backward(torch.empty_like(qd), torch.empty_like(qd), torch.empty_like(qd), torch.zeros(H, W, device="cuda"),
+                                 qd, kd, vd, out, dd, lse, rpb.cuda(), None, B, H, 128, C, W, L, 1.0, workspace=small)
+
+
 def test_deterministic_mode_is_refused_where_it_cannot_be_honoured():
     """Wide windows have no fixed-order reduction of d rpb: asking for one raises instead of falling back to
     atomics without a word."""
@@ -546,6 +619,50 @@ def test_profile_events_bracket_the_kernel():
     assert torch.equal(again, want)
     hip.hipEventDestroy(a)
     hip.hipEventDestroy(b)
+
+
+def test_profile_events_are_refused_under_capture_and_record_nothing():
+    """With a pair of events set, a launch on a capturing stream comes back as NA1D_ERR_LAUNCH and the graph stays
+    empty - the reduction kernel that follows the backward's main launch included."""
+    import ctypes
+    hip = ctypes.CDLL("libamdhip64.so")
+    lib = _lib.load()
+    N, H, T, C, W, L = 4, 4, 100, 16, 27, 13
+    B = N * H
+    q, k, v, do = dev(*make_inputs(B, T, C, W, 4, torch.bfloat16, n=4))
+    rpb = torch.zeros(H, W, device="cuda")
+    out, lse = torch.empty_like(q), torch.empty(B, T, device="cuda")
+    _lib.call_fused_forward(out, lse, q, k, v, rpb, None, B, H, T, C, W, L, 1.0)
+    dq, dk, dv, drpb = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q), torch.zeros(H, W, device="cuda")
+    ws = torch.empty(_lib.fused_backward_workspace_bytes(B, H, T, C, W, L, q.dtype), dtype=torch.uint8, device="cuda")
+    a, b = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    torch.cuda.synchronize()
+    stream = ctypes.c_void_p(side.cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    graph = ctypes.c_void_p()
+    assert hip.hipStreamBeginCapture(stream, 2) == 0          # relaxed mode: other threads of the process are left alone
+    try:
+        assert lib.na1d_profile_events(a, b) == 0
+        st = lib.na1d_fused_backward(P(dq), P(dk), P(dv), P(drpb), P(q), P(k), P(v), P(out), P(do), P(lse), P(rpb), None,
+                                     B, H, T, C, W, L, 1.0, _lib.dtype_tag(q.dtype), P(ws), ws.numel(), stream)
+    finally:
+        lib.na1d_profile_events(None, None)
+        assert hip.hipStreamEndCapture(stream, ctypes.byref(graph)) == 0
+    assert st == -7
+    count = ctypes.c_size_t(99)
+    assert hip.hipGraphGetNodes(graph, None, ctypes.byref(count)) == 0
+    assert count.value == 0
+    hip.hipGraphDestroy(graph)
+    hip.hipEventDestroy(a)
+    hip.hipEventDestroy(b)
+    # the stream is usable again and an ordinary launch on it works
+    with torch.cuda.stream(side):
+        _lib.call_fused_backward(dq, dk, dv, drpb, q, k, v, out, do, lse, rpb, None, B, H, T, C, W, L, 1.0, workspace=ws)
+    side.synchronize()
+    assert torch.isfinite(dq.float()).all()
 
 
 def test_runs_on_the_current_stream():
