@@ -128,7 +128,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
 
     const f32x4 bias_x = {win.bias_x[0], win.bias_x[1], win.bias_x[2], win.bias_x[3]};
     const f32x4 bias_y = {win.bias_y[0], win.bias_y[1], win.bias_y[2], win.bias_y[3]};
-    const float mask_x = kMaskValue * inv_scale;     // the model's additive -100, before the scale
+    const EdgeMask edge = make_edge_mask<DT>(kMaskValue * inv_scale, g);     // the model's additive -100, before the scale
     const int strip_tiles = i1 - i0;
 #pragma unroll
     for (int jt = 0; jt < (MT + TW - 1) / TW; ++jt) {
@@ -147,6 +147,14 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
             read_rows<C>(kop, k_mine + tile_bytes + vb * LL::kTileBytes, k_lane);
             s[vb] = dot_rows_mma<DT, C>(kop, qt, vb == 1 ? bias_y : bias_x);
         }
+        // additive -100 of the model's mask, only on tiles that touch an edge
+        const int s0 = 16 * i - shift;           // first row of the window
+        const int qrow = 16 * i + n;
+        float lse_shift = 0.f;                   // a padded row's logits all carry the -100: its log-sum-exp does too
+        if (s0 < 0 || s0 + 16 * NBV > tv) {
+            add_edge_mask<DT, NBV>(s, edge, s0 + n, qrow, tv);
+            lse_shift = qrow >= tv ? kMaskValue : 0.f;
+        }
         float zx[4], zy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -154,22 +162,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
             zy[r] = s[1][r];
         }
 
-        // additive -100 of the model's mask, only on tiles that touch an edge
-        const int s0 = 16 * i - shift;           // first row of the window
-        const int qrow = 16 * i + n;
-        if (s0 < 0 || s0 + 16 * NBV > tv) {
-            const uint32_t tve = qrow >= tv ? 0u : (uint32_t)tv;     // a padded query row masks all of its slots
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const uint32_t key_y = (uint32_t)(s0 + 16 + 4 * g + r);
-                const uint32_t key_x = (uint32_t)(s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0));
-                zx[r] += key_x >= tve ? mask_x : 0.f;   // unsigned: also key < 0
-                zy[r] += key_y >= tve ? mask_x : 0.f;
-            }
-        }
-
-        float m = max3(max3(zx[0], zx[1], zx[2]), max3(zx[3], zy[0], zy[1]), max2(zy[2], zy[3]));
-        m = xor_max(m);
+        const float m = xor_max(max8_of_accumulators(zx, zy));
         const float nm = -m * scale2;
 
         // The row sums that normalise the output come from the matrix core: a product of the rounded probabilities
@@ -227,7 +220,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
-        const float lse_row = (__builtin_amdgcn_logf(sum) - nm) * kLn2;
+        const float lse_row = __builtin_fmaf(__builtin_amdgcn_logf(sum) - nm, kLn2, lse_shift);
         if (HG > 1 && out_grouped) {          // into the place of this head's Q tile, which only this wave has read
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct)
@@ -429,7 +422,6 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // as in the forward: the accumulators start at rpb / scale, z = x * scale * log2(e) - lse is one multiply-add
     const float scale2 = scale * kLog2e;
     const float inv_scale = __builtin_amdgcn_rcpf(scale);
-    const float mask_x = kMaskValue * inv_scale;
 
     RowLane<C> key_lane, qry_lane;      // row operands: virtual key block rows / query tile rows
     TrLane<C> key_tr, qry_tr;           // transposed operands of the same
@@ -459,6 +451,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     barrier_lds();
     const f32x4 bias_x = {win.bias_x[0], win.bias_x[1], win.bias_x[2], win.bias_x[3]};
     const f32x4 bias_y = {win.bias_y[0], win.bias_y[1], win.bias_y[2], win.bias_y[3]};
+    const EdgeMask edge = make_edge_mask<DT>(kMaskValue * inv_scale, g);
 
     // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
@@ -484,7 +477,13 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             s[vb] = dot_rows_mma<DT, C>(kop, qop, vb == 1 ? bias_y : bias_x);
             dp[vb] = dot_rows_mma<DT, C>(vop, gop);
         }
-        const float nlse2 = -lse_lds[tq * 16 + n] * kLog2e;
+        float nlse2 = -lse_lds[tq * 16 + n] * kLog2e;
+        const int s0 = 16 * qt - shift;
+        const int qrow = 16 * qt + n;
+        if (s0 < 0 || s0 + 16 * NBV > tv) {
+            add_edge_mask<DT, NBV>(s, edge, s0 + n, qrow, tv);
+            if (qrow >= tv) nlse2 += kMaskValue * kLog2e;     // a padded row's log-sum-exp carries the -100 its scores do not
+        }
         float zx[4], zy[4], dpx[4], dpy[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -492,18 +491,6 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             dpx[r] = NBV == 3 ? (win.from0[r] ? dp[0][r] : dp[NBV - 1][r]) : dp[0][r];
             dpy[r] = dp[1][r];
             zy[r] = s[1][r];
-        }
-        const int s0 = 16 * qt - shift;
-        const int qrow = 16 * qt + n;
-        if (s0 < 0 || s0 + 16 * NBV > tv) {
-            const uint32_t tve = qrow >= tv ? 0u : (uint32_t)tv;     // a padded query row masks all of its slots
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const uint32_t key_y = (uint32_t)(s0 + 16 + 4 * g + r);
-                const uint32_t key_x = (uint32_t)(s0 + 4 * g + r + ((NBV == 3 && !win.from0[r]) ? 32 : 0));
-                zx[r] += key_x >= tve ? mask_x : 0.f;   // unsigned: also key < 0
-                zy[r] += key_y >= tve ? mask_x : 0.f;
-            }
         }
         float px[4], py[4], part = 0.f;
 #pragma unroll

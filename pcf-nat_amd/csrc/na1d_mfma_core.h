@@ -277,6 +277,17 @@ __device__ inline float max3(float a, float b, float c) {
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
     return r;
 }
+// Maximum of eight values that may come straight out of matrix-core accumulators.  The compiler keeps the wait
+// states between a matrix instruction and a vector instruction that reads its result, but it cannot see into inline
+// assembly, so the block brings its own: up to 11 idle states are owed after the widest product used here (16x16x32).
+__device__ inline float max8_of_accumulators(const float (&x)[4], const float (&y)[4]) {
+    float a, b, c;
+    asm("s_nop 7\n\ts_nop 3\n\t"
+        "v_max3_f32 %0, %3, %4, %5\n\tv_max3_f32 %1, %6, %7, %8\n\tv_max_f32 %2, %9, %10\n\tv_max3_f32 %0, %0, %1, %2"
+        : "=&v"(a), "=&v"(b), "=&v"(c)
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(y[0]), "v"(y[1]), "v"(y[2]), "v"(y[3]));
+    return a;
+}
 __device__ inline float xor_max(float x) {
     float a, b;
     swap_rows16(x, a, b);
@@ -370,6 +381,39 @@ __device__ inline void read_window(Window<NBV> &w, LDS_PTR(float) tab, int L, in
     }
     w.keep0 = u32x2{m[0] | (m[1] << 16), m[2] | (m[3] << 16)};
     w.keep2 = u32x2{~w.keep0.x, ~w.keep0.y};
+}
+
+// ---- the model's additive mask on edge tiles --------------------------------------------
+// A score gets the reference's -100 when its key lies outside [0, tv) and its query row is a valid one; a padded
+// query row (row >= tv) has all of its slots masked there, a uniform shift that the softmax does not see, so it gets
+// none here.  That makes the mask a product a[key] * b[query] - a = 1 on keys outside the range, b = -100 / scale on
+// valid rows - and the matrix core adds it to a block's scores with one more instruction per block: a sits in
+// channels 0 and 1 of a 16-channel operand, b as a 16-bit value and the rounding error of that value in the same two
+// channels (their sum is -100 / scale to 2^-16).  Three vector instructions per block instead of four per score slot.
+struct EdgeMask {
+    uint32_t hi_lo;      // b's two channels, packed; 0 in the lanes that hold other channels (g != 0)
+    uint32_t one2;       // two ones in the operand's type
+};
+template <class DT> __device__ inline EdgeMask make_edge_mask(float mask_x, int g) {
+    // a half-precision operand cannot hold less than -65504: scales below 100 / 65504 get the largest mask it can
+    const float m = DT::tag == NA1D_FP16 ? __builtin_fmaxf(mask_x, -60000.f) : mask_x;
+    const uint32_t hi = Mma<DT>::pack(m, 0.f) & 0xffffu;
+    const float hi_f = DT::tag == NA1D_BF16 ? __uint_as_float(hi << 16) : (float)__builtin_bit_cast(_Float16, (uint16_t)hi);
+    const uint32_t lo = Mma<DT>::pack(m - hi_f, 0.f) & 0xffffu;
+    return EdgeMask{g == 0 ? (hi | (lo << 16)) : 0u, DT::tag == NA1D_BF16 ? 0x3f803f80u : 0x3c003c00u};
+}
+// s[vb] += mask for the NBV key blocks of a tile whose first key row is key0 - n (key0 = that row + this lane's n).
+template <class DT, int NBV>
+__device__ inline void add_edge_mask(f32x4 (&s)[NBV], const EdgeMask &e, int key0, int qrow, int tv) {
+    const u32x2 b = {qrow < tv ? e.hi_lo : 0u, 0u};
+    uint32_t a[NBV];
+#pragma unroll
+    for (int vb = 0; vb < NBV; ++vb) {
+        a[vb] = (uint32_t)(key0 + 16 * vb) >= (uint32_t)tv ? e.one2 : 0u;      // unsigned: also key < 0
+        settle(a[vb]);
+    }
+#pragma unroll
+    for (int vb = 0; vb < NBV; ++vb) s[vb] = Mma<DT>::k16(u32x2{a[vb], 0u}, b, s[vb]);
 }
 
 // A wave-uniform int32 through the scalar cache: it does not count on the vector-memory counter, so waiting for it
