@@ -182,8 +182,9 @@ int na1d_fused_backward_strided(void *dq, void *dk, void *dv, float *drpb,
  *     mix32(x): x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16   (32-bit arithmetic)
  * and kept probabilities are scaled by 1 / (1 - p_drop); lse is that of the un-dropped softmax.  The mask is a pure
  * function of (seed, b, t, j): the backward recomputes it from the same p_drop and seed, nothing is stored, and the
- * stream differs from torch's (whose mask depends on its launch geometry).  0 <= p_drop < 1.  head_dim > 128
- * returns NA1D_ERR_UNSUPPORTED for p_drop > 0.  Dilated windows: na1d_fused_forward_strided_dropout.  All other arguments as in na1d_fused_forward / na1d_fused_backward.
+ * stream differs from torch's (whose mask depends on its launch geometry).  0 <= p_drop < 1.  Every head_dim the
+ * plain entry points take is covered (above 128 by the generic kernels).  Dilated windows:
+ * na1d_fused_forward_strided_dropout.  All other arguments as in na1d_fused_forward / na1d_fused_backward.
  */
 int na1d_fused_forward_dropout(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
                                const int32_t *t_valid, int64_t B, int64_t H, int64_t T, int64_t C, int64_t W,
@@ -285,9 +286,8 @@ int64_t na1d_fused_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int
  * (no hipMalloc / hipFree, no allocating library routine).  Results are bit-identical to na1d_fused_backward given
  * a workspace of na1d_fused_backward_workspace_bytes() bytes.
  *
- * Limits: the shape must be one the workspace path covers (head_dim <= 128, W <= 32 with at most 16 keys on
- * either side; otherwise NA1D_ERR_UNSUPPORTED), and na1d_fused_backward_workspace_bytes() for it must not exceed
- * NA1D_NOALLOC_SCRATCH_BYTES (32768 workgroups), otherwise NA1D_ERR_TOO_LARGE.  All calls on one GPU share that
+ * Limits: the shape must be one the workspace path covers (head_dim <= 128; otherwise NA1D_ERR_UNSUPPORTED), and na1d_fused_backward_workspace_bytes() for it must not exceed
+ * NA1D_NOALLOC_SCRATCH_BYTES (32768 workgroups; 13107 with windows the wide kernels serve), otherwise NA1D_ERR_TOO_LARGE.  All calls on one GPU share that
  * GPU's array: calls that overlap in time on one GPU (different streams or threads) race on it; calls on one
  * stream are ordered and safe.  The array needs no clearing between calls: a call writes every entry it reads.
  * The device that owns `stream` must be the current device.  The first call on a device looks the array's address

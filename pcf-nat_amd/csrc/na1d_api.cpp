@@ -97,7 +97,8 @@ int mfma_fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, con
     const int st = na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, in, outl, scale,
                                          dtype, workspace, workspace_bytes, s);
     if (st != NA1D_ERR_UNSUPPORTED) return st;
-    return na1d::mfma::wide_bwd(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, dtype, s);
+    return na1d::mfma::wide_bwd(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, dtype, workspace,
+                                workspace_bytes, s);
 }
 
 int band_qk(void *attn, const void *a, const void *b, const Geom &g, int dtype, hipStream_t s) {
@@ -379,8 +380,8 @@ int na1d_fused_backward_noalloc(void *dq, void *dk, void *dv, float *drpb, const
     const int ss = na1d::mfma::static_scratch(&scratch);
     if (ss != NA1D_OK) return ss;
     const na1d::Layout packed = na1d::packed_layout(g);
-    return na1d::mfma::fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, packed, packed, scale,
-                                 dtype, scratch, need, (hipStream_t)stream);
+    return mfma_fused_bwd(dq, dk, dv, drpb, q, k, v, out, dout, lse, rpb, t_valid, g, packed, packed, scale, dtype, scratch,
+                          need, (hipStream_t)stream);
 }
 
 int64_t na1d_global_backward_workspace_bytes(int64_t B, int64_t H, int64_t T, int64_t C, int dtype) {

@@ -182,7 +182,8 @@ int wide_fwd(void *out, float *lse, const void *q, const void *k, const void *v,
              int dtype, hipStream_t s);
 int wide_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v, const void *dout,
              const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g, const Layout &in,
-             const Layout &out_layout, float scale, int dtype, hipStream_t s);
+             const Layout &out_layout, float scale, int dtype, float *workspace, int64_t workspace_bytes, hipStream_t s);
+int64_t wide_bwd_workspace_bytes(const Geom &g);               // 0 when the shape is not covered
 // Dense attention over whole sequences (the models' global layers); g.W and g.L are not used.
 int global_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,
                const Geom &g, float scale, int dtype, hipStream_t s);

@@ -119,7 +119,7 @@ __global__ void __launch_bounds__(kThreads)
 fused_fwd_kernel(Chunk8 *__restrict__ out, float *__restrict__ lse, const Chunk8 *__restrict__ q,
                  const Chunk8 *__restrict__ k, const Chunk8 *__restrict__ v, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, int64_t rows, int64_t T, int C8, int W, int L, int H,
-                 float scale) {
+                 float scale, Dropout drop) {
     extern __shared__ float z[];   // [kFwdRows][W]
     const int64_t r0 = (int64_t)blockIdx.x * kFwdRows;
     const int nr = (int)((rows - r0) < kFwdRows ? (rows - r0) : kFwdRows);
@@ -152,7 +152,12 @@ fused_fwd_kernel(Chunk8 *__restrict__ out, float *__restrict__ lse, const Chunk8
         }
         const float inv = 1.0f / sum;
         for (int j = 0; j < W; ++j) zr[j] *= inv;
-        if (lse) lse[r0 + threadIdx.x] = m + __logf(sum);
+        if (lse) lse[r0 + threadIdx.x] = m + __logf(sum);          // of the softmax before any probability is dropped
+        if (drop.threshold) {                                          // the keep rule of na1d_common.h, slot by slot
+            const int64_t row = r0 + threadIdx.x, b = row / T;
+            const uint32_t key = dropout_row_key(dropout_row(drop, (uint64_t)b, (int)T, (int)(row - b * T)), drop);
+            for (int j = 0; j < W; ++j) zr[j] = dropout_keeps(key, j, drop) ? zr[j] * drop.inv_keep : 0.f;
+        }
     }
     __syncthreads();
 
@@ -187,7 +192,7 @@ fused_bwd_kernel(Chunk8 *__restrict__ dq, Chunk8 *__restrict__ dk, Chunk8 *__res
                  const Chunk8 *__restrict__ v, const Chunk8 *__restrict__ o, const Chunk8 *__restrict__ go,
                  const float *__restrict__ lse, const float *__restrict__ rpb,
                  const int32_t *__restrict__ t_valid, int64_t T, int tiles, int R, int C8, int W, int L, int H,
-                 float scale) {
+                 float scale, Dropout drop) {
     extern __shared__ float smem[];
     const int Rw = W - 1 - L;
     const int E = R + W - 1;
@@ -225,7 +230,15 @@ fused_bwd_kernel(Chunk8 *__restrict__ dq, Chunk8 *__restrict__ dk, Chunk8 *__res
             }
             const float zz = logit_of(s, scale, rpb_h, j, t >= tv || u < 0 || u >= tv);
             p = fast_exp(zz - lse[base + t]);
-            ds = p * (dp - delta[e]);
+            if (drop.threshold) {      // O = (D * P) V with D = 0 or 1 / (1 - p_drop): dP carries D, and so does the P that dV sees
+                const uint32_t key = dropout_row_key(dropout_row(drop, (uint64_t)b, (int)T, (int)t), drop);
+                const float f = dropout_keeps(key, j, drop) ? drop.inv_keep : 0.f;
+                dp *= f;
+                ds = p * (dp - delta[e]);      // delta = rowsum(dO * O) is that of the dropped output already
+                p *= f;
+            } else {
+                ds = p * (dp - delta[e]);
+            }
         }
         P[idx] = p;
         dS[idx] = ds;
@@ -310,21 +323,19 @@ int gather(void *out, const float *attn, const void *x, const Geom &g, int dtype
 
 int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const float *rpb,
               const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s) {
-    if (g.drop.threshold) return NA1D_ERR_UNSUPPORTED;      // dropout lives in the matrix-core kernels only
     const int64_t rows = g.B * g.T;
     const int64_t blocks = (rows + kFwdRows - 1) / kFwdRows;
     if (blocks > 0x7fffffffLL) return NA1D_ERR_SHAPE;
     const size_t smem = (size_t)kFwdRows * g.W * sizeof(float);
     NA1D_BY_DTYPE((fused_fwd_kernel<DT><<<(unsigned)blocks, kThreads, smem, s>>>(
         (Chunk8 *)out, lse, (const Chunk8 *)q, (const Chunk8 *)k, (const Chunk8 *)v, rpb, t_valid, rows, g.T,
-        g.C / 8, g.W, g.L, g.H, scale)));
+        g.C / 8, g.W, g.L, g.H, scale, g.drop)));
     return launch_status();
 }
 
 int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
               const void *out, const void *dout, const float *lse, const float *rpb,
               const int32_t *t_valid, const Geom &g, float scale, int dtype, hipStream_t s) {
-    if (g.drop.threshold) return NA1D_ERR_UNSUPPORTED;
     int R = 32;
     auto bytes = [&](int r) { return (size_t)(2 * (r + g.W - 1) * g.W + (r + g.W - 1)) * sizeof(float); };
     while (R > 8 && bytes(R) > 60 * 1024) R /= 2;
@@ -334,7 +345,7 @@ int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const vo
     NA1D_BY_DTYPE((fused_bwd_kernel<DT><<<(unsigned)blocks, kThreads, bytes(R), s>>>(
         (Chunk8 *)dq, (Chunk8 *)dk, (Chunk8 *)dv, drpb, (const Chunk8 *)q, (const Chunk8 *)k, (const Chunk8 *)v,
         (const Chunk8 *)out, (const Chunk8 *)dout, lse, rpb, t_valid, g.T, (int)tiles, R, g.C / 8, g.W, g.L, g.H,
-        scale)));
+        scale, g.drop)));
     return launch_status();
 }
 

@@ -315,27 +315,6 @@ int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v
 //     second evaluation of the scores.
 // d rpb partial sums: one row of kPartialStride floats per work item, folded in a
 // fixed order by a second kernel (one workgroup per head).
-constexpr int kPartialStride = 32;
-
-__global__ void __launch_bounds__(128)
-drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, int N, int H, int strips, int W) {
-    __shared__ float acc[128];
-    const int h = blockIdx.x / W, j = blockIdx.x - h * W;
-    const int rows = N * strips;                      // items of this head: (n, strip)
-    float s = 0.f;
-    for (int i = threadIdx.x; i < rows; i += 128) {
-        const int n = i / strips, st = i - n * strips;
-        s += partial[((size_t)(n * H + h) * strips + st) * kPartialStride + j];
-    }
-    acc[threadIdx.x] = s;
-    __syncthreads();
-    for (int half = 64; half > 0; half >>= 1) {       // fixed tree: the result does not depend on timing
-        if ((int)threadIdx.x < half) acc[threadIdx.x] += acc[threadIdx.x + half];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) drpb[h * W + j] += acc[0];
-}
-
 // Waves per SIMD the register allocation of the backward must leave room for.  16-channel heads: the LDS footprint
 // admits six workgroups per CU, so the registers must too (80 or fewer; the dropout variant would spill and is left alone).
 constexpr int bwd_min_waves(int C, bool drop) { return C == 16 && !drop ? 6 : 1; }
@@ -706,7 +685,7 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                   div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g), g.drop);
     // not behind a launch that was refused (events set on a capturing stream): the sums it would fold do not exist
     if (partial && drpb && !launch_events().refused)
-        drpb_reduce_kernel<<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
+        drpb_reduce_kernel<kPartialStride><<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);
     return launch_status();
 }
 
@@ -726,7 +705,7 @@ int fused_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const vo
 }
 
 int64_t fused_bwd_workspace_bytes(const Geom &g, int dtype) {
-    if (!window_blocks(g)) return 0;
+    if (!window_blocks(g)) return wide_bwd_workspace_bytes(g);     // 0 where the wide kernels do not cover the shape either
     switch (padded_width(g.C)) {   // the split does not depend on the dtype
         case 16: return bwd_workspace<BF16, 16>(g);
         case 32: return bwd_workspace<BF16, 32>(g);

@@ -504,6 +504,32 @@ __device__ inline uint32_t xcd_item(uint32_t wg, uint32_t items) {
     return (wg & 7) * per + (wg >> 3);
 }
 
+// ---- fixed-order reduction of the bias gradient ----------------------------------------
+// With a workspace the backward kernels write one row of STRIDE floats per workgroup (its sums over the window
+// slots) instead of adding them to d rpb with float atomics; this kernel, one workgroup per (head, slot), then folds
+// the rows of a head in a fixed order.
+constexpr int kPartialStride = 32;          // windows of the two/three-block kernels: W <= 32
+constexpr int kWidePartialStride = 80;      // wide windows: W <= 80
+template <int STRIDE>
+__global__ void __launch_bounds__(128)
+drpb_reduce_kernel(float *__restrict__ drpb, const float *__restrict__ partial, int N, int H, int strips, int W) {
+    __shared__ float acc[128];
+    const int h = blockIdx.x / W, j = blockIdx.x - h * W;
+    const int rows = N * strips;                      // items of this head: (n, strip)
+    float s = 0.f;
+    for (int i = threadIdx.x; i < rows; i += 128) {
+        const int n = i / strips, st = i - n * strips;
+        s += partial[((size_t)(n * H + h) * strips + st) * STRIDE + j];
+    }
+    acc[threadIdx.x] = s;
+    __syncthreads();
+    for (int half = 64; half > 0; half >>= 1) {       // fixed tree: the result does not depend on timing
+        if ((int)threadIdx.x < half) acc[threadIdx.x] += acc[threadIdx.x + half];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) drpb[h * W + j] += acc[0];
+}
+
 // While profiling events are set, the launchers note which kernel they are about to launch, spelt as a profiler's
 // kernel trace prints it without namespaces and arguments, e.g. fused_bwd_kernel<FP16, 32, 2, false>.
 inline void note_kernel(const char *base, int dtype, int C, int nbv, int drop = -1, int hg = 0) {

@@ -237,13 +237,13 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
                 const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                 const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
                 const int32_t *__restrict__ t_valid, uint32_t items, int T, int W, int L, int H, int tiles, int nt,
-                int strips, float scale, int kv_bytes, uint32_t strips_magic, uint32_t heads_magic, Strides in,
-                Strides outl, int shift, Dropout drop) {
+                int strips, float scale, float *__restrict__ drpb_partial, int kv_bytes, uint32_t strips_magic,
+                uint32_t heads_magic, Strides in, Strides outl, int shift, Dropout drop) {
     using LL = Lds<C>;
     constexpr int CT = C / 16;
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
     fetch_args_now(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale,
-                   kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width, outl.sample,
+                   drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width, outl.sample,
                    outl.head, outl.pitch, outl.width, shift);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
     const int hb = NBV - 1 - (shift >> 4), ha = (shift + 15) >> 4;
@@ -266,7 +266,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
-    const uint32_t b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
+    const uint32_t item = wi.item, b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
     const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
     const int q0 = i0 - hb;                                 // first query-side tile
@@ -467,7 +467,10 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
         float t = 0.f;
 #pragma unroll
         for (int w = 0; w < kWaves; ++w) t += rsum[w * kWideSlots + 32 + tid];
-        atomicAdd(drpb + head * W + tid, t);
+        if (drpb_partial)
+            drpb_partial[(size_t)item * kWidePartialStride + tid] = t;   // folded by drpb_reduce_kernel
+        else
+            atomicAdd(drpb + head * W + tid, t);
     }
 }
 
@@ -480,47 +483,88 @@ inline size_t wide_bwd_lds(int nt, int nbv, const WideBwdShape &w, int &kv_bytes
            (kThreads + kBiasSlots + kWaves * kWideSlots) * sizeof(float);
 }
 
+// The split of a wide backward into workgroups: strips as long as a CU's LDS allows.
+template <int C>
+inline bool wide_bwd_split(const Geom &g, const WideCover &c, Split &sp, int &kv_bytes, size_t &lds) {
+    const WideBwdShape w = wide_bwd_shape(c);
+    int mt = w.mt;
+    while (mt >= 1 && wide_bwd_lds<C>(mt, c.nbv, w, kv_bytes) > 160 * 1024) --mt;   // LDS of one CU
+    if (mt < 1) return false;
+    sp = make_split(g.B, g.T, mt);
+    lds = wide_bwd_lds<C>(sp.nt, c.nbv, w, kv_bytes);
+    return true;
+}
+
 template <class DT, int C, int NBV>
 int launch_wide_bwd_n(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
                       const void *dout, const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g,
-                      const Layout &in, const Layout &outl, float scale, const WideCover &c, hipStream_t s) {
-    const WideBwdShape w = wide_bwd_shape(c);
-    int mt = w.mt, kv_bytes = 0;
-    while (mt >= 1 && wide_bwd_lds<C>(mt, NBV, w, kv_bytes) > 160 * 1024) --mt;   // LDS of one CU
-    if (mt < 1) return NA1D_ERR_UNSUPPORTED;
-    const Split sp = make_split(g.B, g.T, mt);
+                      const Layout &in, const Layout &outl, float scale, const WideCover &c, float *workspace,
+                      int64_t workspace_bytes, hipStream_t s) {
+    Split sp;
+    int kv_bytes = 0;
+    size_t lds = 0;
+    if (!wide_bwd_split<C>(g, c, sp, kv_bytes, lds)) return NA1D_ERR_UNSUPPORTED;
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
+    float *partial = nullptr;          // as in the two/three-block backward: a workspace is used or refused
+    if (drpb && workspace) {
+        if (workspace_bytes < sp.items * kWidePartialStride * (int64_t)sizeof(float)) return NA1D_ERR_WORKSPACE;
+        partial = workspace;
+    }
     auto kern = g.drop.threshold ? wide_bwd_kernel<DT, C, NBV, true> : wide_bwd_kernel<DT, C, NBV, false>;
-    const size_t lds = wide_bwd_lds<C>(sp.nt, NBV, w, kv_bytes);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     note_kernel("wide_bwd_kernel", DT::tag, C, NBV, g.drop.threshold != 0);
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
-                  g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, kv_bytes, div_magic(sp.strips), div_magic(g.H),
+                  g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips), div_magic(g.H),
                   byte_strides(in, g), byte_strides(outl, g), c.shift, g.drop);
+    if (partial && drpb && !launch_events().refused)
+        drpb_reduce_kernel<kWidePartialStride><<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H,
+                                                                                     sp.strips, g.W);
     return launch_status();
 }
 
 template <class DT, int C>
 int launch_wide_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v,
                     const void *dout, const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g,
-                    const Layout &in, const Layout &outl, float scale, hipStream_t s) {
+                    const Layout &in, const Layout &outl, float scale, float *workspace, int64_t workspace_bytes,
+                    hipStream_t s) {
     const WideCover c = wide_cover(g);
     switch (c.nbv) {
-        case 3: return launch_wide_bwd_n<DT, C, 3>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, s);
-        case 4: return launch_wide_bwd_n<DT, C, 4>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, s);
-        case 5: return launch_wide_bwd_n<DT, C, 5>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, s);
-        case 6: return launch_wide_bwd_n<DT, C, 6>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, s);
+        case 3: return launch_wide_bwd_n<DT, C, 3>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, workspace, workspace_bytes, s);
+        case 4: return launch_wide_bwd_n<DT, C, 4>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, workspace, workspace_bytes, s);
+        case 5: return launch_wide_bwd_n<DT, C, 5>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, workspace, workspace_bytes, s);
+        case 6: return launch_wide_bwd_n<DT, C, 6>(dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, c, workspace, workspace_bytes, s);
     }
     return NA1D_ERR_UNSUPPORTED;
 }
 
-// d rpb is summed with float atomics (there is no workspace path for wide windows).
+// d rpb: float atomics, or - given a workspace of wide_bwd_workspace_bytes() - per-workgroup partial rows that a second
+// kernel folds in a fixed order.
 int wide_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const void *k, const void *v, const void *dout,
              const float *lse, const float *rpb, const int32_t *t_valid, const Geom &g, const Layout &in,
-             const Layout &outl, float scale, int dtype, hipStream_t s) {
+             const Layout &outl, float scale, int dtype, float *workspace, int64_t workspace_bytes, hipStream_t s) {
     if (!wide_cover(g).nbv) return NA1D_ERR_UNSUPPORTED;
-    NA1D_MFMA_DISPATCH(launch_wide_bwd, dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, s);
+    NA1D_MFMA_DISPATCH(launch_wide_bwd, dq, dk, dv, drpb, q, k, v, dout, lse, rpb, t_valid, g, in, outl, scale, workspace,
+                       workspace_bytes, s);
+}
+
+template <int C> int64_t wide_workspace(const Geom &g, const WideCover &c) {
+    Split sp;
+    int kv_bytes = 0;
+    size_t lds = 0;
+    if (!wide_bwd_split<C>(g, c, sp, kv_bytes, lds)) return 0;
+    return sp.items * kWidePartialStride * (int64_t)sizeof(float);
+}
+int64_t wide_bwd_workspace_bytes(const Geom &g) {
+    const WideCover c = wide_cover(g);
+    if (!c.nbv) return 0;
+    switch (padded_width(g.C)) {
+        case 16: return wide_workspace<16>(g, c);
+        case 32: return wide_workspace<32>(g, c);
+        case 64: return wide_workspace<64>(g, c);
+        case 128: return wide_workspace<128>(g, c);
+    }
+    return 0;
 }
 
 }  // namespace mfma

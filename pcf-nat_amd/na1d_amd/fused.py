@@ -28,12 +28,14 @@ def _strided_or_packed_forward(out4, lse, q4, k4, v4, rpb, t_valid, W, left, sca
     ``None`` or ``(p, seed, row_stride, row_offset, seq_rows)``."""
     if _lib.call_fused_forward_strided(out4, lse, q4, k4, v4, rpb, t_valid, W, left, scale, dropout=dropout) == 0:
         return None
-    if dropout is not None:
-        raise _lib.NA1DError("attention dropout needs head_dim <= 128 (no dropout on the generic kernels)")
+    if dropout is not None and len(dropout) > 2 and tuple(dropout[2:4]) != (1, 0):
+        raise _lib.NA1DError("attention dropout with dilated windows needs head_dim <= 128 (the packed entry points "
+                             "name rows by their place in the tensor they are given)")
     N, H, T, C = q4.shape
     qp, kp, vp = (z.contiguous().view(N * H, T, C) for z in (q4, k4, v4))
     op = torch.empty_like(qp)
-    _lib.call_fused_forward(op, lse, qp, kp, vp, rpb, t_valid, N * H, H, T, C, W, left, scale)
+    _lib.call_fused_forward(op, lse, qp, kp, vp, rpb, t_valid, N * H, H, T, C, W, left, scale,
+                            dropout=None if dropout is None else dropout[:2])
     out4.copy_(op.view(N, H, T, C))
     return op
 
@@ -49,7 +51,7 @@ def _strided_or_packed_backward(dq4, dk4, dv4, drpb, q4, k4, v4, packed_out, dou
     qp, kp, vp, gp = (z.contiguous().view(N * H, T, C) for z in (q4, k4, v4, dout4))
     dqp, dkp, dvp = torch.empty_like(qp), torch.empty_like(kp), torch.empty_like(vp)
     _lib.call_fused_backward(dqp, dkp, dvp, drpb, qp, kp, vp, packed_out, gp, lse, rpb, t_valid, N * H, H, T, C, W, left,
-                             scale, workspace=ws)
+                             scale, workspace=ws, dropout=None if dropout is None else dropout[:2])
     for dst, src in ((dq4, dqp), (dk4, dkp), (dv4, dvp)):
         dst.copy_(src.view(N, H, T, C))
 
@@ -65,14 +67,12 @@ def _deterministic_workspace_bytes(B, H, T, C, win_size, left, dilation, dtype):
 
 
 def _deterministic_workspace(B, H, T, C, win_size, left, like, dilation=1):
-    """Scratch for the fixed-order reduction of the bias gradient.  Only the two/three-block matrix-core backward
-    has that path; for the shapes it does not cover (wide windows, head_dim > 128) the library would fall back to
-    float atomics silently, so the request is refused instead."""
+    """Scratch for the fixed-order reduction of the bias gradient.  The matrix-core backward kernels have that path;
+    for head_dim > 128 (the generic kernels) the library would use float atomics, so the request is refused instead."""
     nbytes = _deterministic_workspace_bytes(B, H, T, C, win_size, left, dilation, like.dtype)
     if nbytes <= 0:
-        raise _lib.NA1DError("deterministic=True: no fixed-order reduction of the bias gradient for head_dim %d, "
-                             "window %d (left %d); it covers head_dim <= 128 and windows of at most 32 slots with "
-                             "at most 16 on either side" % (C, win_size, left))
+        raise _lib.NA1DError("deterministic=True: no fixed-order reduction of the bias gradient for head_dim %d "
+                             "(it covers head_dim <= 128)" % C)
     return torch.empty(nbytes, dtype=torch.uint8, device=like.device)
 
 

@@ -89,6 +89,7 @@ def test_fused_entry_points_validate():
     assert w(4096, 16, 100, 16, 27, 13, 0) == 4096 * 32 * 4      # one 32-float row per work item
     assert w(1024, 8, 300, 32, 15, 7, 1) > 0
     assert w(4, 2, 8, 136, 5, 2, 0) == 0                         # generic kernel: no workspace
+    assert w(64, 2, 300, 32, 65, 32, 0) > 0 and w(64, 2, 300, 32, 65, 32, 0) % (80 * 4) == 0   # wide windows: rows of 80 floats
     assert w(4, 3, 8, 16, 5, 2, 0) == -5 and w(4, 2, 8, 16, 99, 2, 0) == -4
 
 
@@ -102,7 +103,7 @@ def test_noalloc_entry_point_validates_and_respects_the_kernel_family_switch():
                          kw.get("C", 16), kw.get("W", 5), 2, kw.get("scale", 1.0), 0, None]
     assert f(*args(lse=None)) == -1 and f(*args(C=20)) == -3 and f(*args(W=99)) == -4 and f(*args(scale=0.0)) == -11
     assert f(*args(B=0)) == 0                        # nothing to do
-    assert f(*args(C=136)) == -8 and f(*args(W=40)) == -8        # shapes without a fixed-order reduction
+    assert f(*args(C=136)) == -8                     # head_dim above 128: the generic kernels have no fixed-order reduction
     assert f(*args(B=1 << 20)) == -9                 # more workgroups than the static scratch holds rows for
     was = lib.na1d_force_generic(1)
     try:
@@ -156,7 +157,6 @@ def test_dropout_entry_points_validate():
                          kw.get("p", 0.5), 7, None]
     assert f(*args(v=None)) == -1 and f(*args(C=20)) == -3 and f(*args(B=0)) == 0
     assert f(*args(p=1.0)) == -5 and f(*args(p=-0.1)) == -5 and f(*args(p=float("nan"))) == -5
-    assert f(*args(C=136)) == -8                     # no dropout kernel above head_dim 128
     b = lib.na1d_fused_backward_dropout
     bargs = lambda **kw: [ok, ok, ok, None, ok, ok, ok, ok, ok, kw.get("lse", ok), None, None, 4, 2, 8, 16, 5, 2, 1.0, 0,
                           kw.get("p", 0.5), 7, None, 0, None]

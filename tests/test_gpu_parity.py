@@ -508,9 +508,9 @@ def test_deterministic_rpb_gradient_with_dilated_windows():
 
 
 def test_deterministic_mode_is_refused_where_it_cannot_be_honoured():
-    """Wide windows have no fixed-order reduction of d rpb: asking for one raises instead of falling back to
-    atomics without a word."""
-    N, H, T, C, W, L = 2, 2, 80, 16, 33, 16
+    """Heads wider than 128 channels run the generic kernels, which have no fixed-order reduction of d rpb: asking
+    for one raises instead of falling back to atomics without a word."""
+    N, H, T, C, W, L = 2, 2, 40, 136, 9, 4
     q, k, v, do = make_inputs(N * H, T, C, W, 72, torch.float16, n=4, scale=0.25)
     qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
     rd = (torch.randn(H, W) * 0.3).cuda().requires_grad_(True)
@@ -519,6 +519,27 @@ def test_deterministic_mode_is_refused_where_it_cannot_be_honoured():
         out.backward(do.cuda())
     na1d_fused(qd, kd, vd, W, L, rpb=rd, num_heads=H).backward(do.cuda())          # the default still works
     assert torch.isfinite(rd.grad).all()
+
+
+@pytest.mark.parametrize("geom", [(8, 4, 150, 32, 33, 16), (4, 2, 200, 16, 65, 32), (3, 2, 90, 64, 80, 0)],
+                         ids=lambda g: "x".join(map(str, g)))
+def test_deterministic_rpb_gradient_with_wide_windows(geom):
+    """The wide-window backward folds d rpb in a fixed order too, given a workspace: two runs give the same bits and
+    the atomics path agrees to fp32 rounding."""
+    N, H, T, C, W, L = geom
+    q, k, v, do = make_inputs(N * H, T, C, W, 74, torch.bfloat16, n=4, scale=C ** -0.5)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(7)) * 0.3
+    grads = []
+    for det in (True, True, False):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        rd = rpb.cuda().requires_grad_(True)
+        na1d_fused(qd, kd, vd, W, L, rpb=rd, num_heads=H, deterministic=det).backward(do.cuda())
+        grads.append((rd.grad.clone(), qd.grad.clone(), kd.grad.clone(), vd.grad.clone()))
+    assert all(torch.equal(a, b) for a, b in zip(grads[0], grads[1]))
+    assert all(torch.equal(a, b) for a, b in zip(grads[0][1:], grads[2][1:]))
+    assert torch.allclose(grads[0][0], grads[2][0], rtol=1e-4, atol=1e-4)
+    want = O.na1d_backward(q.float(), k.float(), v.float(), do.float(), W, L, rpb, None, H)[3]
+    assert _err(grads[0][0].cpu(), want) < TOL[torch.bfloat16]
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
@@ -691,6 +712,7 @@ def test_errors_become_python_exceptions():
 DROP_GEOMS = [  # (N, H, T, C, W, L): two-block, merged three-block, wide and lopsided windows, padded head dims, ragged tiles
     (2, 2, 61, 32, 15, 7), (2, 4, 100, 16, 27, 13), (1, 2, 150, 64, 33, 16), (2, 1, 90, 32, 65, 32),
     (2, 2, 47, 24, 9, 0), (1, 3, 130, 128, 17, 16), (2, 2, 5, 16, 27, 13), (1, 2, 300, 48, 80, 50),
+    (2, 2, 40, 136, 9, 4), (1, 2, 70, 160, 27, 13),      # heads wider than 128 channels: the generic kernels
 ]
 
 
@@ -834,10 +856,9 @@ def test_dropout_rate_zero_is_the_plain_operator_and_bad_rates_are_rejected():
     out = torch.empty_like(q)
     with pytest.raises(_lib.NA1DError):
         _lib.call_fused_forward(out, None, q, k, v, None, None, 4, 1, 50, 32, 15, 7, 1.0, dropout=(1.0, 1))
-    wide = torch.zeros(2, 8, 136, dtype=torch.bfloat16, device="cuda")
-    with pytest.raises(_lib.NA1DError):                               # head_dim > 128 has no dropout kernels
-        _lib.call_fused_forward(torch.empty_like(wide), None, wide, wide, wide, None, None, 2, 1, 8, 136, 5, 2, 1.0,
-                                dropout=(0.5, 1))
+    wide = torch.randn(2, 9, 3, 1, 136, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).cuda()
+    with pytest.raises(_lib.NA1DError, match="dilated"):              # head_dim > 128: dropout, but not on dilated windows
+        na1d_fused_qkv(wide.requires_grad_(True), 5, 2, dilation=2, dropout_p=0.5, seed=1)
 
 
 def test_inference_path_of_the_projection_layout_equals_the_autograd_path():

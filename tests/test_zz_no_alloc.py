@@ -63,6 +63,7 @@ def test_no_alloc_backward_matches_the_workspace_backward_twice():
     _backward_both_ways(64, 8, 300, 32, 15, 7, torch.float16, seed=1, first_on_device=True)
     _backward_both_ways(3, 4, 90, 16, 27, 13, torch.bfloat16, seed=2, pad=[0, 30, 90])
     _backward_both_ways(5, 2, 40, 48, 9, 4, torch.float16, seed=3)          # head_dim run at the next kernel width
+    _backward_both_ways(6, 4, 150, 32, 65, 32, torch.bfloat16, seed=4, pad=[0, 0, 20, 150, 3, 77])   # wide window
 
 
 def test_no_alloc_backward_replays_from_a_captured_graph():
@@ -120,6 +121,6 @@ def test_no_alloc_backward_limits():
     # more workgroups than the scratch array has rows for: refused before anything is launched
     assert f(ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, None, 1 << 16, 1, 16, 16, 27, 13, 1.0, 0, None) == -9
     assert b"scratch" in lib.na1d_status_string(-9)
-    # a window the workspace path does not cover
-    assert f(ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, None, 4, 1, 64, 16, 65, 32, 1.0, 0, None) == -8
+    # a head_dim the workspace path does not cover
+    assert f(ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, ok, None, 4, 1, 64, 136, 27, 13, 1.0, 0, None) == -8
     assert f(ok, ok, ok, ok, ok, ok, ok, ok, ok, None, ok, None, 4, 1, 64, 16, 27, 13, 1.0, 0, None) == -1
