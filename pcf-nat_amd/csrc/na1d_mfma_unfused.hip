@@ -65,7 +65,7 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     constexpr int MT = kBandMaxTiles;
     fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
     // dynamic LDS: K region of kt tiles starting sb tiles before the strip, Q region of nt tiles, two 16 x W fp32
-    // tiles per wave
+    // tiles per wave and behind them a word per lane for the results that belong to no slot
     const int sb = (shift + 15) >> 4, kt = nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
@@ -96,9 +96,25 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     RowLane<C> k_lane, q_lane;
     k_lane.init(16 * sb - shift, lane);
     q_lane.init(0, lane);
-    LDS_PTR(float) mine = out_lds + wave * 32 * W;
+    LDS_PTR(float) mine = out_lds + wave * (32 * W + 64);
+    // Where this lane's four results of virtual block vb go inside a 16 x W tile: slot j = 16*vb + 4g + r - shift - n + L
+    // of row n, the same for every tile.  Slots outside the window are sent to a word of the lane's own behind the
+    // wave's two tiles, so that every write is unconditional: twelve masked writes a tile, each behind its own
+    // branch, were most of the instructions of a tile.
+    int slot_at[2][NBV][4];             // byte offsets from `mine`, for the first and the second tile of a pair
+#pragma unroll
+    for (int vb = 0; vb < NBV; ++vb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int j = 16 * vb + 4 * g + r - shift - n + L;
+            const bool in_window = j >= 0 && j < W;
+            slot_at[0][vb][r] = (in_window ? n * W + j : 32 * W + lane) * 4;
+            slot_at[1][vb][r] = (in_window ? 16 * W + n * W + j : 32 * W + lane) * 4;
+            settle(slot_at[0][vb][r]);
+            settle(slot_at[1][vb][r]);
+        }
     wait_direct();
-    __syncthreads();
+    barrier_lds();
 
     // A wave takes two neighbouring tiles at a time: their 32*W floats are a run of W whole 128-byte lines (where the
     // sequence's rows start on a line), which leaves as one streaming write instead of two pieces per tile that L2
@@ -108,9 +124,10 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     // is still the faster policy (15.4 against 16.1 us), the two shared lines being a small part of a run's 27.
     for (int i = i0 + 2 * wave; i < i1; i += 2 * kWaves) {
         const int pair = min(2, i1 - i);
-        for (int h = 0; h < pair; ++h) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            if (h >= pair) break;
             const int tile_bytes = (i + h - i0) * LL::kTileBytes;
-            LDS_PTR(float) tile = mine + h * 16 * W;
             RowOperand<C> qt;
             read_rows<C>(qt, q_lds + tile_bytes, q_lane);
 #pragma unroll
@@ -119,10 +136,8 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
                 read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
                 const f32x4 s = dot_rows_mma<DT, C>(kop, qt);
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int j = 16 * vb + 4 * g + r - shift - n + L;
-                    if (j >= 0 && j < W) tile[n * W + j] = s[r];  // every (row, slot) is written by exactly one lane
-                }
+                for (int r = 0; r < 4; ++r)        // every (row, slot) is written by exactly one lane
+                    *reinterpret_cast<LDS_PTR(float)>((LDS_PTR(char))mine + slot_at[h][vb][r]) = s[r];
             }
         }
         // LDS serves one wave's accesses in program order, so the other lanes' values are there when the
@@ -292,7 +307,7 @@ template <class DT, int C, int NBV>
 int launch_qk_n(float *attn, const void *a, const void *b, const Geom &g, const BandCover &c, hipStream_t s) {
     auto lds_of = [&](int nt) {
         return (size_t)region_bytes<C>(nt - 1 + NBV + ((c.shift & 15) ? 1 : 0)) + region_bytes<C>(nt) +
-               (size_t)kWaves * 32 * g.W * sizeof(float);
+               (size_t)kWaves * (32 * g.W + 64) * sizeof(float);
     };
     const int mt = fit_tiles(c.max_tiles, lds_of);
     if (mt < 1) return NA1D_ERR_UNSUPPORTED;
