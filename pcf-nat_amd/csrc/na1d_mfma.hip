@@ -317,7 +317,7 @@ int fused_fwd(void *out, float *lse, const void *q, const void *k, const void *v
 // fixed order by a second kernel (one workgroup per head).
 // Waves per SIMD the register allocation of the backward must leave room for.  16-channel heads: the LDS footprint
 // admits six workgroups per CU, so the registers must too (80 or fewer; the dropout variant would spill and is left alone).
-constexpr int bwd_min_waves(int C, bool drop) { return C == 16 && !drop ? 6 : 1; }
+constexpr int bwd_min_waves(int C, bool drop, bool one) { return C == 16 && !drop ? (one ? 7 : 6) : 1; }
 
 // Rows that no other workgroup reads: the backward takes them with the workgroup-scope policy rather than the
 // non-temporal one of the forward (measured: 4-7 % on the 16-channel backward, nothing either way at 32 channels; the
@@ -327,9 +327,19 @@ constexpr int kBwdMinItems = 256;      // fewer items than this: shorter strips
 template <int C> struct StripBwd {
     static constexpr int kMaxTiles = C <= 32 ? 8 : C <= 64 ? 4 : 2;
 };
+// Floats of the region that first holds the lse of the query-side rows (staged by whole waves, a row per lane) and
+// after pass 1 the waves' 32 d rpb slot sums each.
+__host__ __device__ inline bool bwd_bias_in_padding(int kv_bytes, int key_region) { return kv_bytes - 2 * key_region >= kBiasEntries * (int)sizeof(float); }
+template <int C> constexpr int bwd_lse_rows(bool one) {
+    const int rows = ((StripBwd<C>::kMaxTiles + (one ? 0 : 2)) * 16 + 63) / 64 * 64;
+    return rows > kWaves * 32 ? rows : kWaves * 32;
+}
 
-template <class DT, int C, int NBV, bool DROP>
-__global__ void __launch_bounds__(kThreads, bwd_min_waves(C, DROP))
+// ONE: the strip is the whole sequence (strips == 1).  There are no neighbouring strips then and no halo tiles of
+// queries either side: two tiles fewer in the Q and dO regions and in a wave's share of pass 1, which is what lets a
+// seventh workgroup of 16-channel heads onto a CU (LDS and registers both).
+template <class DT, int C, int NBV, bool DROP, bool ONE>
+__global__ void __launch_bounds__(kThreads, bwd_min_waves(C, DROP, ONE))
 fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, float *__restrict__ drpb,
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
@@ -344,55 +354,58 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                    drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width,
                    outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
-    constexpr int kRowsQ = (MT + 2) * 16;
-    constexpr int TPW = (MT + 2 + kWaves - 1) / kWaves;    // query tiles per wave, at most
+    constexpr int HALO = ONE ? 0 : 1;                      // query tiles either side of the strip whose scores pass 2 needs
+    constexpr int kRowsQ = (MT + 2 * HALO) * 16;
+    constexpr int TPW = (MT + 2 * HALO + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
-    static_assert(kRowsQ <= kThreads, "one lane per staged lse row");
+    constexpr int kLseRows = bwd_lse_rows<C>(ONE);
+    static_assert(kRowsQ <= kLseRows && kLseRows <= kThreads, "one lane per staged lse row");
     // dynamic LDS (see launch_bwd): [K region | V region] of nt+1+NBV tiles each, starting at the first key of
     // query tile i0-1 (row 16*(i0-1) - shift, so that virtual key blocks are whole tiles of the region), reused after
-    // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt+2 tiles (rows 16*i0 - 16 ...); lse
-    // of the query-side rows; the head's bias table; and - only when d rpb is wanted - 32 slot sums per wave
+    // pass 1 for the score tiles and padded to kv_bytes; Q, dO regions of nt + 2*HALO tiles (rows 16*(i0 - HALO) ...); lse
+    // of the query-side rows, whose place the 32 d rpb slot sums per wave take after pass 1; the head's bias table
+    // where the padding of the K/V regions has no room for it
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int key_region = region_bytes<C>(nt + 1 + NBV), qry_region = region_bytes<C>(nt + 2);
+    const int key_region = region_bytes<C>(nt + 1 + NBV), qry_region = region_bytes<C>(nt + 2 * HALO);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
-    LDS_PTR(char) sc_lds = k_lds;                  // score tiles [((tq - sc_skip)*2 + X/Y)*2 + P/dS]
+    LDS_PTR(char) sc_lds = k_lds;                  // score tiles [(tq*2 + X/Y)*2 + P/dS], tq = query tile - (i0 - HALO)
     LDS_PTR(char) q_lds = k_lds + kv_bytes;
     LDS_PTR(char) g_lds = q_lds + qry_region;      // dO
     LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + qry_region);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    LDS_PTR(float) bias_lds = lse_lds + kThreads;                           // the head's bias table
-    LDS_PTR(float) rsum = lse_lds + kThreads + kBiasEntries;                // [kWaves][32] d rpb slot sums per wave
+    // the head's bias table, read before pass 1 only: in what the score tiles need beyond the K and V regions, if that is room enough
+    LDS_PTR(float) bias_lds = bwd_bias_in_padding(kv_bytes, key_region) ? (LDS_PTR(float))(k_lds + 2 * key_region) : lse_lds + kLseRows;
+    LDS_PTR(float) rsum = lse_lds;                                          // [kWaves][32] d rpb slot sums per wave, once every wave has read its lse
     const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
     const uint32_t item = wi.item, b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
     const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
     const int g = lane >> 4, n = lane & 15;
-    const int sc_skip = strips == 1 ? 1 : 0;       // a strip that is the whole sequence has no halo tiles to keep scores of
 
     const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
     BiasTable bias_raw;
     load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
     {
         const int key_bytes = min(T, 16 * (i1 + 2)) * in.pitch;
-        const int qry_rows = min(T, 16 * (i1 + 1));
+        const int qry_rows = min(T, 16 * (i1 + HALO));
         const Rsrc ks = make_rsrc(k + in_off, key_bytes), vs = make_rsrc(v + in_off, key_bytes);
         const Rsrc qs = make_rsrc(q + in_off, qry_rows * in.pitch), gs = make_rsrc(dout + out_off, qry_rows * outl.pitch);
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
         const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
         const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch, outl.width);
         // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
-        load_to_lds<4, 0>(ls, (LDS_PTR(char))(lse_lds + 64 * wave), (16 * i0 - 16 + tid) * 4);
-        if (strips == 1 && (in.pitch == 2 * C || C % 64 == 0) && (outl.pitch == 2 * C || C % 64 == 0)) {
+        if (64 * wave < kRowsQ) load_to_lds<4, 0>(ls, (LDS_PTR(char))(lse_lds + 64 * wave), (16 * (i0 - HALO) + tid) * 4);
+        if (ONE && (in.pitch == 2 * C || C % 64 == 0) && (outl.pitch == 2 * C || C % 64 == 0)) {
             stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadOnceBwd>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2 * HALO, kReadOnceBwd>(qs, 16 * (i0 - HALO), q_lds, nt + 2 * HALO, wave, lane_off, in.pitch);
             stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadOnceBwd>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
+            stage_direct<C, MT + 2 * HALO, kReadOnceBwd>(gs, 16 * (i0 - HALO), g_lds, nt + 2 * HALO, wave, lane_off_g, outl.pitch);
         } else {
             stage_direct<C, MT + 1 + NBV, kReadShared>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadShared>(qs, 16 * i0 - 16, q_lds, nt + 2, wave, lane_off, in.pitch);
+            stage_direct<C, MT + 2 * HALO, kReadShared>(qs, 16 * (i0 - HALO), q_lds, nt + 2 * HALO, wave, lane_off, in.pitch);
             stage_direct<C, MT + 1 + NBV, kReadShared>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
-            stage_direct<C, MT + 2, kReadShared>(gs, 16 * i0 - 16, g_lds, nt + 2, wave, lane_off_g, outl.pitch);
+            stage_direct<C, MT + 2 * HALO, kReadShared>(gs, 16 * (i0 - HALO), g_lds, nt + 2 * HALO, wave, lane_off_g, outl.pitch);
         }
     }
 
@@ -432,7 +445,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     const f32x4 bias_y = {win.bias_y[0], win.bias_y[1], win.bias_y[2], win.bias_y[3]};
     const EdgeMask edge = make_edge_mask<DT>(kMaskValue * inv_scale, g);
 
-    // ---------------- pass 1: query tiles i0-1 .. i1 -> dQ, d rpb, score tiles ----------------
+    // ---------------- pass 1: query tiles i0-HALO .. i1-1+HALO -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
     const Rsrc dqs = make_rsrc(dq + in_off, T * in.pitch);
     const bool dq_whole_lines = stores_whole_lines(in.pitch, C, 0);
@@ -441,8 +454,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     for (int jt = 0; jt < TPW; ++jt) {
         sc[jt][0][0] = sc[jt][0][1] = sc[jt][1][0] = sc[jt][1][1] = u32x2{0u, 0u};
         const int tq = wave + jt * kWaves;                  // tile index inside the query-side regions
-        const int qt = i0 - 1 + tq;
-        if (qt > i1 || qt < 0 || qt >= tiles) continue;     // nothing there: its scores stay zero
+        const int qt = i0 - HALO + tq;
+        if (qt >= i1 + HALO || qt < 0 || qt >= tiles) continue;     // nothing there: its scores stay zero
         RowOperand<C> qop, gop;
         read_rows<C>(qop, q_lds + tq * LL::kTileBytes, qry_lane);
         read_rows<C>(gop, g_lds + tq * LL::kTileBytes, qry_lane);
@@ -511,7 +524,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         sc[jt][1][0] = u32x2{Mma<DT>::pack(py[0], py[1]), Mma<DT>::pack(py[2], py[3])};
         sc[jt][0][1] = u32x2{Mma<DT>::pack(dsx[0], dsx[1]), Mma<DT>::pack(dsx[2], dsx[3])};
         sc[jt][1][1] = u32x2{Mma<DT>::pack(dsy[0], dsy[1]), Mma<DT>::pack(dsy[2], dsy[3])};
-        if (qt < i0 || qt >= i1) continue;                  // halo tile: only its scores are needed
+        if (HALO && (qt < i0 || qt >= i1)) continue;        // halo tile: only its scores are needed
 
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -548,8 +561,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // permutation lines the 16 diagonals a - n = d (mod 16) up in lane d; the two members of a class, a - n = d
     // and a - n = d - 16, are told apart by a >= d and go to slots 16 apart, set X and set Y crosswise.  What is
     // left is a sum over the 16 keys a: four registers, then the four lane groups.  Fixed order throughout.
+    float s0 = 0.f, s1 = 0.f;             // slots (n + L - shift) mod 32 and 16 further, n = this lane's class
     if (drpb) {
-        float s0 = 0.f, s1 = 0.f;         // slots (n + L - shift) mod 32 and 16 further, n = this lane's class
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int a = 4 * g + r;
@@ -562,18 +575,20 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
         s0 = xor_sum(s0);
         s1 = xor_sum(s1);
+    }
+
+    barrier_lds();                    // every wave is done with K, V and lse: their regions become the score tiles and the d rpb sums
+    if (drpb) {
         const int slot = (n + L - shift) & 31;
         if (g == 0) rsum[wave * 32 + slot] = s0;
         if (g == 1) rsum[wave * 32 + ((slot + 16) & 31)] = s1;
     }
-
-    barrier_lds();                    // every wave is done with K and V: their regions become the score tiles
 #pragma unroll
     for (int jt = 0; jt < TPW; ++jt) {
         const int tq = wave + jt * kWaves;
-        const int qt = i0 - 1 + tq;
-        if (qt > i1 || qt < 0 || qt >= tiles) continue;                      // no such tile: pass 2 does not look for it
-        LDS_PTR(char) t = sc_lds + (tq - sc_skip) * 4 * kScoreTile + n * 32 + g * 8;   // tile[query n][key slots 4g..4g+3]
+        const int qt = i0 - HALO + tq;
+        if (qt >= i1 + HALO || qt < 0 || qt >= tiles) continue;              // no such tile: pass 2 does not look for it
+        LDS_PTR(char) t = sc_lds + tq * 4 * kScoreTile + n * 32 + g * 8;   // tile[query n][key slots 4g..4g+3]
 #pragma unroll
         for (int xy = 0; xy < 2; ++xy)
 #pragma unroll
@@ -610,10 +625,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             // that is there and drop what it holds
             const bool there = (uint32_t)(kp - vb) < (uint32_t)tiles;
             const uint32_t tm = there ? 0xffffffffu : 0u;
-            const int tq = kp - vb - (i0 - 1);
+            const int tq = there ? kp - vb - (i0 - HALO) : HALO;       // a tile that is there, whatever it holds
             LDS_PTR(char) qtile = q_lds + tq * LL::kTileBytes;
             LDS_PTR(char) gtile = g_lds + tq * LL::kTileBytes;
-            LDS_PTR(char) stile = sc_lds + (((there ? tq : 1) - sc_skip) * 4 + (vb == 1 ? 2 : 0)) * kScoreTile + sc_lane;
+            LDS_PTR(char) stile = sc_lds + (tq * 4 + (vb == 1 ? 2 : 0)) * kScoreTile + sc_lane;
             u32x2 pb = read_tr(stile), db = read_tr(stile + kScoreTile);
             if (NBV == 3 && vb == 0) {
                 pb = u32x2{pb.x & keep0t.x & tm, pb.y & keep0t.y & tm};
@@ -670,15 +685,22 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
         partial = workspace;
     }
     const bool two = window_blocks(g) == 2;
-    auto kern = g.drop.threshold ? (two ? fused_bwd_kernel<DT, C, 2, true> : fused_bwd_kernel<DT, C, 3, true>)
-                                 : (two ? fused_bwd_kernel<DT, C, 2, false> : fused_bwd_kernel<DT, C, 3, false>);
+    const bool one = sp.strips == 1;
+    auto kern = g.drop.threshold
+                    ? (two ? (one ? fused_bwd_kernel<DT, C, 2, true, true> : fused_bwd_kernel<DT, C, 2, true, false>)
+                           : (one ? fused_bwd_kernel<DT, C, 3, true, true> : fused_bwd_kernel<DT, C, 3, true, false>))
+                    : (two ? (one ? fused_bwd_kernel<DT, C, 2, false, true> : fused_bwd_kernel<DT, C, 2, false, false>)
+                           : (one ? fused_bwd_kernel<DT, C, 3, false, true> : fused_bwd_kernel<DT, C, 3, false, false>));
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
     // (a strip that is the whole sequence has no halo tiles)
-    const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + (sp.strips == 1 ? 0 : 2)) * 4 * 512);
-    const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2) +
-                       (kThreads + kBiasEntries + (drpb ? kWaves * 32 : 0)) * sizeof(float);
+    const int halo = one ? 0 : 1;
+    const int kv_bytes = std::max(2 * region_bytes<C>(sp.nt + 1 + window_blocks(g)), (sp.nt + 2 * halo) * 4 * 512);
+    const bool bias_apart = !bwd_bias_in_padding(kv_bytes, region_bytes<C>(sp.nt + 1 + window_blocks(g)));
+    const size_t lds = (size_t)kv_bytes + (size_t)2 * region_bytes<C>(sp.nt + 2 * halo) +
+                       (bwd_lse_rows<C>(one) + (bias_apart ? kBiasEntries : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    note_kernel("fused_bwd_kernel", DT::tag, C, two ? 2 : 3, g.drop.threshold != 0);
+    note_kernel_as("fused_bwd_kernel<%s, %d, %d, %s, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C, two ? 2 : 3,
+                   g.drop.threshold ? "true" : "false", one ? "true" : "false");
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),

@@ -230,6 +230,23 @@ __device__ inline void read_rows(RowOperand<C> &o, LDS_PTR(char) tile, const Row
     for (int s = 0; s < RowOperand<C>::k32; ++s) o.w32[s] = *reinterpret_cast<LDS_PTR(u32x4)>(tile + l.off32[s]);
     if (RowOperand<C>::k16) o.w16[0] = *reinterpret_cast<LDS_PTR(u32x2)>(tile + l.off16);
 }
+// The same operand straight from memory, for rows that only this wave needs: lane (n, g) asks for its pieces of the
+// row `n` rows behind byte offset `tile` of the resource (rows of `width` bytes, `pitch` bytes apart; pieces past the
+// width, like rows past the resource's end, arrive as zeros).
+template <int C, int AUX>
+__device__ inline void load_rows(RowOperand<C> &o, Rsrc src, int tile, int pitch, int width, int lane) {
+    const int g = lane >> 4, n = lane & 15;
+    const int row = tile + n * pitch;
+#pragma unroll
+    for (int s = 0; s < RowOperand<C>::k32; ++s) {
+        const int at = 64 * s + 16 * g;
+        o.w32[s] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(src, at < width ? row + at : kNowhere, 0, AUX));
+    }
+    if (RowOperand<C>::k16) {
+        const int at = 64 * RowOperand<C>::k32 + 8 * g;
+        o.w16[0] = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(src, at < width ? row + at : kNowhere, 0, AUX));
+    }
+}
 template <class DT, int C>
 __device__ inline f32x4 dot_rows_mma(const RowOperand<C> &a, const RowOperand<C> &b, f32x4 acc = f32x4{0.f, 0.f, 0.f, 0.f}) {
 #pragma unroll

@@ -54,6 +54,12 @@ __device__ inline float score_at(LDS_PTR(float) rows, int row, int j, int W) {  
     return (j >= 0 && j < W) ? val : 0.f;
 }
 
+// Narrow heads and few key blocks: the key rows of a wave's two tiles (NBV + 1 tiles of them) fit its registers as well,
+// and the kernel needs no staged input, no barrier and no wait but each wave's own.
+template <int C, int NBV> constexpr bool qk_keys_direct() { return (NBV + 1) * (C / 8) <= 16; }
+// Whether the K region of kt tiles ends with at least 64 words that its copies fill but no tile uses.
+template <int C> __host__ __device__ constexpr bool qk_spare_words(int kt) { return region_bytes<C>(kt) - kt * Lds<C>::kTileBytes >= 256; }
+
 // =============================================================================
 // P1: attn[b,t,j] = sum_c a[b,t,c] * b~[b,t-L+j,c]
 // =============================================================================
@@ -64,13 +70,12 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     using LL = Lds<C>;
     constexpr int MT = kBandMaxTiles;
     fetch_args_now(attn, qa, kb, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
-    // dynamic LDS: K region of kt tiles starting sb tiles before the strip, Q region of nt tiles, two 16 x W fp32
-    // tiles per wave and behind them a word per lane for the results that belong to no slot
+    // dynamic LDS: K region of kt tiles starting sb tiles before the strip, two 16 x W fp32 tiles per wave (and 64 words for the results that belong to no slot, unless the K region's padding has them)
     const int sb = (shift + 15) >> 4, kt = nt - 1 + NBV + ((shift & 15) ? 1 : 0);
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) q_lds = k_lds + region_bytes<C>(kt);
-    LDS_PTR(float) out_lds = (LDS_PTR(float))(q_lds + region_bytes<C>(nt));
+    constexpr bool kDirect = qk_keys_direct<C, NBV>();
+    LDS_PTR(float) out_lds = (LDS_PTR(float))(k_lds + (kDirect ? 0 : region_bytes<C>(kt)));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -81,26 +86,43 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     const int g = lane >> 4, n = lane & 15;
 
     const int64_t seq_off = (int64_t)b * T * pitch;      // packed rows of head_dim = pitch / 2 channels
+    // A wave computes two neighbouring tiles (a strip has at most eight): their query rows, which no other wave needs,
+    // come straight into the registers of the matrix operand - the key rows, which three tiles share, go through LDS.
+    // Not staging the query rows is worth two more workgroups on a CU at 32 channels.
+    const int i = i0 + 2 * wave;
+    RowOperand<C> qt[2], kr[kDirect ? NBV + 1 : 1];
     {
         const int key_bytes = min(T, 16 * (i0 - sb + kt)) * pitch, qry_bytes = min(T, 16 * i1) * pitch;
         const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
-        if (strips == 1) {      // nobody else reads these rows
+        const Rsrc qs = make_rsrc(qa + seq_off, qry_bytes);
+        if constexpr (kDirect) {
+            const Rsrc ks = make_rsrc(kb + seq_off, T * pitch);
+            // neighbouring waves ask for the same key rows at about the same time: the default policy, whatever the strips
+#pragma unroll
+            for (int j = 0; j <= NBV; ++j) load_rows<C, kReadShared>(kr[j], ks, (16 * (i + j) - shift) * pitch, pitch, pitch, lane);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) load_rows<C, kReadOnce>(qt[h], qs, 16 * (i + h) * pitch, pitch, pitch, lane);
+        } else if (strips == 1) {      // nobody else reads these rows
             stage_direct<C, MT + NBV, kReadOnce>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off, pitch);
-            stage_direct<C, MT, kReadOnce>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off, pitch);
-        } else {                // (the read-once policy on the query rows alone measured 8 % slower at T = 300)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) load_rows<C, kReadOnce>(qt[h], qs, 16 * (i + h) * pitch, pitch, pitch, lane);
+        } else {
             stage_direct<C, MT + NBV, kReadShared>(make_rsrc(kb + seq_off, key_bytes), 16 * (i0 - sb), k_lds, kt, wave, lane_off, pitch);
-            stage_direct<C, MT, kReadShared>(make_rsrc(qa + seq_off, qry_bytes), 16 * i0, q_lds, nt, wave, lane_off, pitch);
+#pragma unroll
+            for (int h = 0; h < 2; ++h) load_rows<C, kReadShared>(qt[h], qs, 16 * (i + h) * pitch, pitch, pitch, lane);
         }
     }
     const Rsrc as = make_rsrc(attn + (int64_t)b * T * W, T * W * 4);
-    RowLane<C> k_lane, q_lane;
+    RowLane<C> k_lane;
     k_lane.init(16 * sb - shift, lane);
-    q_lane.init(0, lane);
-    LDS_PTR(float) mine = out_lds + wave * (32 * W + 64);
+    LDS_PTR(float) mine = out_lds + wave * 32 * W;
     // Where this lane's four results of virtual block vb go inside a 16 x W tile: slot j = 16*vb + 4g + r - shift - n + L
-    // of row n, the same for every tile.  Slots outside the window are sent to a word of the lane's own behind the
-    // wave's two tiles, so that every write is unconditional: twelve masked writes a tile, each behind its own
-    // branch, were most of the instructions of a tile.
+    // of row n, the same for every tile.  Slots outside the window are sent to a word per lane that nobody reads (one
+    // set of 64 words for all waves: in the padding of the K region where the copies leave that much, else behind the
+    // waves' tiles), so that every write is unconditional: twelve masked writes a tile, each behind its own branch,
+    // were most of the instructions of a tile.
+    const int nowhere = (int)(!kDirect && qk_spare_words<C>(kt) ? (LDS_PTR(char))k_lds + kt * LL::kTileBytes - (LDS_PTR(char))mine
+                                                     : (LDS_PTR(char))(out_lds + kWaves * 32 * W) - (LDS_PTR(char))mine) + lane * 4;
     int slot_at[2][NBV][4];             // byte offsets from `mine`, for the first and the second tile of a pair
 #pragma unroll
     for (int vb = 0; vb < NBV; ++vb)
@@ -108,13 +130,15 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
         for (int r = 0; r < 4; ++r) {
             const int j = 16 * vb + 4 * g + r - shift - n + L;
             const bool in_window = j >= 0 && j < W;
-            slot_at[0][vb][r] = (in_window ? n * W + j : 32 * W + lane) * 4;
-            slot_at[1][vb][r] = (in_window ? 16 * W + n * W + j : 32 * W + lane) * 4;
+            slot_at[0][vb][r] = in_window ? (n * W + j) * 4 : nowhere;
+            slot_at[1][vb][r] = in_window ? (16 * W + n * W + j) * 4 : nowhere;
             settle(slot_at[0][vb][r]);
             settle(slot_at[1][vb][r]);
         }
-    wait_direct();
-    barrier_lds();
+    if constexpr (!kDirect) {
+        wait_direct();
+        barrier_lds();
+    }
 
     // A wave takes two neighbouring tiles at a time: their 32*W floats are a run of W whole 128-byte lines (where the
     // sequence's rows start on a line), which leaves as one streaming write instead of two pieces per tile that L2
@@ -122,19 +146,21 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
     // line (T*W*4 not a multiple of 128: the run then shares its first and last line with the neighbouring runs) and
     // for the single last tile: measured with 100 rows of 27 slots, where no sequence but the first is aligned, it
     // is still the faster policy (15.4 against 16.1 us), the two shared lines being a small part of a run's 27.
-    for (int i = i0 + 2 * wave; i < i1; i += 2 * kWaves) {
+    static_assert(kBandMaxTiles <= 2 * kWaves, "a wave's two tiles cover the strip");
+    if (i < i1) {
         const int pair = min(2, i1 - i);
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
             if (h >= pair) break;
             const int tile_bytes = (i + h - i0) * LL::kTileBytes;
-            RowOperand<C> qt;
-            read_rows<C>(qt, q_lds + tile_bytes, q_lane);
 #pragma unroll
             for (int vb = 0; vb < NBV; ++vb) {
                 RowOperand<C> kop;
-                read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
-                const f32x4 s = dot_rows_mma<DT, C>(kop, qt);
+                if constexpr (kDirect)
+                    kop = kr[h + vb];
+                else
+                    read_rows<C>(kop, k_lds + tile_bytes + vb * LL::kTileBytes, k_lane);
+                const f32x4 s = dot_rows_mma<DT, C>(kop, qt[h]);
 #pragma unroll
                 for (int r = 0; r < 4; ++r)        // every (row, slot) is written by exactly one lane
                     *reinterpret_cast<LDS_PTR(float)>((LDS_PTR(char))mine + slot_at[h][vb][r]) = s[r];
@@ -147,8 +173,6 @@ qk_kernel(float *__restrict__ attn, const char *__restrict__ qa, const char *__r
         const int first = 16 * i * W;                             // floats into the sequence's score rows
         for (int u = lane; u * 4 < pair * 16 * W; u += 64)
             __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<LDS_PTR(u32x4)>(mine + u * 4), as, (first + u * 4) * 4, 0, kStoreAux);
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");    // tiles read before the next pair overwrites them
-        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -306,8 +330,10 @@ inline int fit_tiles(int max_tiles, F lds_of) {
 template <class DT, int C, int NBV>
 int launch_qk_n(float *attn, const void *a, const void *b, const Geom &g, const BandCover &c, hipStream_t s) {
     auto lds_of = [&](int nt) {
-        return (size_t)region_bytes<C>(nt - 1 + NBV + ((c.shift & 15) ? 1 : 0)) + region_bytes<C>(nt) +
-               (size_t)kWaves * (32 * g.W + 64) * sizeof(float);
+        const int kt = nt - 1 + NBV + ((c.shift & 15) ? 1 : 0);
+        const bool direct = qk_keys_direct<C, NBV>();
+        return (size_t)(direct ? 0 : region_bytes<C>(kt)) + (size_t)kWaves * 32 * g.W * sizeof(float) +
+               (!direct && qk_spare_words<C>(kt) ? 0 : 64 * sizeof(float));
     };
     const int mt = fit_tiles(c.max_tiles, lds_of);
     if (mt < 1) return NA1D_ERR_UNSUPPORTED;
