@@ -24,6 +24,10 @@ SHAPES = [
     (2, 100, 128, 80, 39), (2, 17, 16, 80, 0), (2, 130, 64, 7, 3), (4, 300, 32, 15, 7), (3, 65, 16, 27, 26),
     (2, 47, 48, 33, 16), (2, 64, 16, 27, 13), (1, 16, 32, 15, 7), (2, 15, 64, 7, 3), (2, 250, 16, 9, 8),
     (2, 70, 56, 27, 13), (1, 90, 72, 15, 7), (2, 50, 96, 40, 20), (1, 33, 120, 7, 3), (2, 40, 136, 9, 4),
+    # the QK kernel's two forms side by side: key rows straight into registers (head_dim 16 with any window, head_dim
+    # 32 up to three key blocks) and through LDS (head_dim 32 from four key blocks on), ragged and whole last tile pairs
+    (3, 128, 16, 80, 40), (2, 113, 16, 49, 48), (2, 100, 32, 27, 13), (2, 129, 32, 33, 0), (3, 97, 24, 40, 20),
+    (2, 144, 8, 17, 16),
 ]
 
 
@@ -138,6 +142,9 @@ FUSED_GEOMS = [  # (N, H, T, C, W, left)
     (3, 4, 150, 16, 27, 13), (2, 8, 300, 32, 15, 7), (4, 4, 200, 64, 7, 3), (1, 2, 129, 128, 5, 2), (2, 2, 48, 16, 1, 0),
     (1, 4, 257, 32, 40, 7), (1, 2, 31, 64, 33, 20), (2, 2, 90, 56, 27, 13), (1, 2, 75, 72, 15, 7), (2, 1, 60, 96, 50, 25),
     (1, 2, 40, 120, 7, 3), (2, 2, 100, 8, 27, 13), (1, 2, 50, 136, 9, 4),
+    # either side of the backward's single-strip form (a strip of at most eight tiles that is the whole sequence)
+    (2, 2, 128, 16, 27, 13), (1, 3, 128, 32, 15, 7), (2, 2, 127, 32, 9, 4), (1, 2, 113, 16, 17, 16), (1, 2, 129, 16, 27, 13),
+    (2, 1, 64, 64, 7, 3), (1, 2, 65, 64, 15, 7), (1, 1, 32, 128, 5, 2), (1, 2, 16, 16, 27, 13),
 ]
 
 
