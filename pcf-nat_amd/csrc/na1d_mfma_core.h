@@ -162,9 +162,9 @@ __device__ inline int direct_lane_offset(int wave, int lane, int pitch = Lds<C>:
     return unit * 16 < width ? (lane / Lds<C>::kUnits) * pitch + unit * 16 : kNowhere;
 }
 // One wave-wide load that writes LDS directly: lane l's BYTES (4 or 16) land at lds + BYTES * l.  Written out by hand
-// so that the compiler knows nothing of it: told of such loads it puts waits for ALL of them in front of LDS reads it
-// cannot tell apart from their target, which defeats copies that are issued early and waited for in parts.  Callers
-// wait with wait_direct() before they (or, behind a barrier, other waves) read the target.
+// so that the compiler knows nothing of it: told of such loads it puts a wait for ALL loads in flight in front of every
+// LDS read it cannot tell apart from their target (the bias table, for one), and so serialises what was issued early
+// on purpose.  Callers wait with wait_direct() before they (or, behind a barrier, other waves) read the target.
 template <int BYTES, int AUX>
 __device__ inline void load_to_lds(Rsrc src, LDS_PTR(char) lds, int offset) {
     static_assert((BYTES == 4 || BYTES == 16) && (AUX == 0 || AUX == 1 || AUX == 2 || AUX == 3), "load size / cache policy");
@@ -191,6 +191,23 @@ __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, 
     for (int j = 0; j < kRounds; ++j) {
         const int c = j * NW + wave;
         if (c < chunks) load_to_lds<16, AUX>(src, region + c * kChunk, base + c * step);
+    }
+}
+// The same into a region of exactly `bytes` bytes (a multiple of 16) that is not padded to whole chunks: the last chunk
+// is loaded by as many lanes as it has 16-byte units, so nothing is written behind the region and another region can
+// follow it directly.  LDS is granted in units of 1280 bytes; the kilobyte or so of padding that two regions carry can
+// be the difference between seven and eight workgroups on a CU.
+template <int AUX, int ROUNDS, int NW = kWaves, class OFFSET>
+__device__ inline void stage_exact(Rsrc src, LDS_PTR(char) region, int bytes, int wave, int lane, OFFSET offset_of_chunk) {
+    const int whole = bytes / kChunk, tail = bytes - whole * kChunk;
+#pragma unroll
+    for (int j = 0; j < ROUNDS; ++j) {
+        const int c = j * NW + wave;
+        if (c < whole) {
+            load_to_lds<16, AUX>(src, region + c * kChunk, offset_of_chunk(c));
+        } else if (c == whole && lane * 16 < tail) {       // only these lanes take part: the others' units do not exist
+            load_to_lds<16, AUX>(src, region + c * kChunk, offset_of_chunk(c));
+        }
     }
 }
 __device__ inline void wait_direct() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }

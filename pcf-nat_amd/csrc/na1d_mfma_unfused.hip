@@ -255,11 +255,11 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     fetch_args_now(out, attn, x, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
     // Key block kp (rows 16*kp - shift ...) is virtual block vb of query tile kp - vb, so the blocks that touch the
     // strip's rows need the query tiles i0 - hb .. i1 - 1 + ha.  Dynamic LDS: their x rows (qtiles tiles) and their
-    // score rows (qtiles*16 x W fp32)
+    // score rows (qtiles*16 x W fp32), neither padded to whole copy chunks (stage_exact)
     const int hb = NBV - 1 - (shift >> 4), ha = (shift + 15) >> 4, qtiles = nt + hb + ha;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) x_lds = (LDS_PTR(char))smem;
-    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + region_bytes<C>(qtiles));
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + qtiles * LL::kTileBytes);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -274,12 +274,19 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     {
         const int rows_hi = min(T, 16 * (q0 + qtiles));
         const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
+        const Rsrc xs = make_rsrc(x + seq_off, rows_hi * pitch), ss = make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4);
+        constexpr int kRowRounds = (region_bytes<C>(MT + NBV) / kChunk + kWaves - 1) / kWaves;
+        constexpr int kScoreRounds = (((kBandMaxTiles + NBV) * 16 * (16 * NBV - 15) * 4 + kChunk - 1) / kChunk + kWaves - 1) / kWaves;
+        const int x_first = 16 * q0 * pitch + lane_off, x_step = (kChunk / LL::kRowBytes) * pitch;
+        const int s_first = 16 * q0 * W * 4 + lane * 16;
+        auto x_at = [&](int c) { return x_first + c * x_step; };
+        auto s_at = [&](int c) { return s_first + c * kChunk; };
         if (strips == 1) {      // nobody else reads these rows
-            stage_direct<C, MT + NBV, kReadOnce>(make_rsrc(x + seq_off, rows_hi * pitch), 16 * q0, x_lds, qtiles, wave, lane_off, pitch);
-            stage_scores<NBV, kReadOnce>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), 16 * q0 * W, s_lds, qtiles, W, wave, lane);
+            stage_exact<kReadOnce, kRowRounds>(xs, x_lds, qtiles * LL::kTileBytes, wave, lane, x_at);
+            stage_exact<kReadOnce, kScoreRounds>(ss, (LDS_PTR(char))s_lds, qtiles * 16 * W * 4, wave, lane, s_at);
         } else {
-            stage_direct<C, MT + NBV, kReadShared>(make_rsrc(x + seq_off, rows_hi * pitch), 16 * q0, x_lds, qtiles, wave, lane_off, pitch);
-            stage_scores<NBV, kReadShared>(make_rsrc(attn + (int64_t)b * T * W, rows_hi * W * 4), 16 * q0 * W, s_lds, qtiles, W, wave, lane);
+            stage_exact<kReadShared, kRowRounds>(xs, x_lds, qtiles * LL::kTileBytes, wave, lane, x_at);
+            stage_exact<kReadShared, kScoreRounds>(ss, (LDS_PTR(char))s_lds, qtiles * 16 * W * 4, wave, lane, s_at);
         }
     }
     TrLane<C> x_tr;
@@ -369,7 +376,7 @@ int launch_av_n(void *out, const float *attn, const void *v, const Geom &g, cons
 template <class DT, int C, int NBV>
 int launch_gather_n(void *out, const float *attn, const void *x, const Geom &g, const BandCover &c, hipStream_t s) {
     const int halo = NBV - 1 - (c.shift >> 4) + ((c.shift + 15) >> 4);          // query tiles beyond the strip
-    auto lds_of = [&](int nt) { return (size_t)region_bytes<C>(nt + halo) + score_bytes(nt + halo, g.W); };
+    auto lds_of = [&](int nt) { return (size_t)(nt + halo) * Lds<C>::kTileBytes + (size_t)(nt + halo) * 16 * g.W * 4; };
     const int mt = fit_tiles(c.max_tiles, lds_of);
     if (mt < 1) return NA1D_ERR_UNSUPPORTED;
     const Split sp = make_split(g.B, g.T, mt);
