@@ -242,6 +242,8 @@ av_kernel(char *__restrict__ out, const float *__restrict__ attn, const char *__
     }
 }
 
+template <int C> constexpr bool gather_exact_regions() { return C == 16; }
+
 // =============================================================================
 // P3: out[b,u,c] = sum_j attn[b,u+L-j,j] * x[b,u+L-j,c]
 // =============================================================================
@@ -255,11 +257,14 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
     fetch_args_now(out, attn, x, items, T, W, L, tiles, nt, strips, strips_magic, shift, pitch);
     // Key block kp (rows 16*kp - shift ...) is virtual block vb of query tile kp - vb, so the blocks that touch the
     // strip's rows need the query tiles i0 - hb .. i1 - 1 + ha.  Dynamic LDS: their x rows (qtiles tiles) and their
-    // score rows (qtiles*16 x W fp32), neither padded to whole copy chunks (stage_exact)
+    // score rows (qtiles*16 x W fp32); at 16 channels, where a tile is half a copy chunk and the padding of the two
+    // regions is what stands between seven and eight workgroups on a CU, neither is padded to whole chunks
+    // (stage_exact; wider heads gain no workgroup by it and lose 1-2 % to the shorter last copy)
+    constexpr bool kExact = gather_exact_regions<C>();
     const int hb = NBV - 1 - (shift >> 4), ha = (shift + 15) >> 4, qtiles = nt + hb + ha;
     extern __shared__ __attribute__((aligned(16))) char smem[];
     LDS_PTR(char) x_lds = (LDS_PTR(char))smem;
-    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + qtiles * LL::kTileBytes);
+    LDS_PTR(float) s_lds = (LDS_PTR(float))(x_lds + (kExact ? qtiles * LL::kTileBytes : region_bytes<C>(qtiles)));
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -281,12 +286,20 @@ gather_kernel(char *__restrict__ out, const float *__restrict__ attn, const char
         const int s_first = 16 * q0 * W * 4 + lane * 16;
         auto x_at = [&](int c) { return x_first + c * x_step; };
         auto s_at = [&](int c) { return s_first + c * kChunk; };
-        if (strips == 1) {      // nobody else reads these rows
-            stage_exact<kReadOnce, kRowRounds>(xs, x_lds, qtiles * LL::kTileBytes, wave, lane, x_at);
-            stage_exact<kReadOnce, kScoreRounds>(ss, (LDS_PTR(char))s_lds, qtiles * 16 * W * 4, wave, lane, s_at);
+        if constexpr (kExact) {
+            if (strips == 1) {      // nobody else reads these rows
+                stage_exact<kReadOnce, kRowRounds>(xs, x_lds, qtiles * LL::kTileBytes, wave, lane, x_at);
+                stage_exact<kReadOnce, kScoreRounds>(ss, (LDS_PTR(char))s_lds, qtiles * 16 * W * 4, wave, lane, s_at);
+            } else {
+                stage_exact<kReadShared, kRowRounds>(xs, x_lds, qtiles * LL::kTileBytes, wave, lane, x_at);
+                stage_exact<kReadShared, kScoreRounds>(ss, (LDS_PTR(char))s_lds, qtiles * 16 * W * 4, wave, lane, s_at);
+            }
+        } else if (strips == 1) {
+            stage_direct<C, MT + NBV, kReadOnce>(xs, 16 * q0, x_lds, qtiles, wave, lane_off, pitch);
+            stage_scores<NBV, kReadOnce>(ss, 16 * q0 * W, s_lds, qtiles, W, wave, lane);
         } else {
-            stage_exact<kReadShared, kRowRounds>(xs, x_lds, qtiles * LL::kTileBytes, wave, lane, x_at);
-            stage_exact<kReadShared, kScoreRounds>(ss, (LDS_PTR(char))s_lds, qtiles * 16 * W * 4, wave, lane, s_at);
+            stage_direct<C, MT + NBV, kReadShared>(xs, 16 * q0, x_lds, qtiles, wave, lane_off, pitch);
+            stage_scores<NBV, kReadShared>(ss, 16 * q0 * W, s_lds, qtiles, W, wave, lane);
         }
     }
     TrLane<C> x_tr;
@@ -376,7 +389,10 @@ int launch_av_n(void *out, const float *attn, const void *v, const Geom &g, cons
 template <class DT, int C, int NBV>
 int launch_gather_n(void *out, const float *attn, const void *x, const Geom &g, const BandCover &c, hipStream_t s) {
     const int halo = NBV - 1 - (c.shift >> 4) + ((c.shift + 15) >> 4);          // query tiles beyond the strip
-    auto lds_of = [&](int nt) { return (size_t)(nt + halo) * Lds<C>::kTileBytes + (size_t)(nt + halo) * 16 * g.W * 4; };
+    auto lds_of = [&](int nt) {
+        return gather_exact_regions<C>() ? (size_t)(nt + halo) * Lds<C>::kTileBytes + (size_t)(nt + halo) * 16 * g.W * 4
+                                         : (size_t)region_bytes<C>(nt + halo) + score_bytes(nt + halo, g.W);
+    };
     const int mt = fit_tiles(c.max_tiles, lds_of);
     if (mt < 1) return NA1D_ERR_UNSUPPORTED;
     const Split sp = make_split(g.B, g.T, mt);
