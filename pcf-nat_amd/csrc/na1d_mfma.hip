@@ -18,7 +18,11 @@ constexpr int kGroupWaves = 8;               // waves per workgroup when heads a
 // can be staged together: the strip copies then move HG * C channels of a row in one piece - whole 128-byte lines
 // for four heads of 16 channels, where a head alone would ask for quarter lines - into regions laid out as rows of
 // C * HG channels, and every wave computes the tiles of one head (kGroupWaves / HG waves share a head's tiles).
-template <class DT, int C, int NBV, bool DROP, int HG>
+// ONE: one head per workgroup (HG == 1) and the strip is the whole sequence.  Nothing is shared with another workgroup
+// then, and what a workgroup works out before its first copy can go - strip arithmetic, the XCD-aware order - is cut to
+// the sample / head split and three buffer resources: at T around 100 a launch is one round of workgroups, and every
+// instruction in front of the first copy is in the launch's duration (6 ns apiece, measured by adding some).
+template <class DT, int C, int NBV, bool DROP, int HG, bool ONE>
 __global__ void __launch_bounds__(64 * (HG > 1 ? kGroupWaves : kWaves))
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
@@ -32,6 +36,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     constexpr int CT = C / 16;                       // channel tiles of the output
     constexpr int MT = HG > 1 ? kGroupTiles : Strip<CS>::kMaxTiles;
     static_assert(NW % HG == 0, "whole waves per head");
+    static_assert(!ONE || HG == 1, "the whole-sequence form is for single heads");
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
@@ -47,24 +52,34 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + region_bytes<CS>(nt)) + (HG > 1 ? wave % HG : 0) * kBiasEntries;   // the bias table of this wave's head
-    const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H / HG, heads_magic);
     const int hw = HG > 1 ? wave % HG : 0;           // this wave's head inside the group
-    const uint32_t sample = wi.sample, head0 = wi.head * HG, head = head0 + hw, b = sample * H + head;
-    const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
+    uint32_t sample, head0;
+    int i0, i1;
+    if constexpr (ONE) {
+        // heads that interleave in memory share lines: their workgroups stay on one XCD, behind one L2 (xcd_item);
+        // packed rows are nobody else's, and the plain order is 3 % faster
+        const uint32_t lin = in.pitch == 2 * C && outl.pitch == 2 * C ? blockIdx.x : xcd_item(blockIdx.x, items);
+        sample = div_by(lin, H, heads_magic);
+        head0 = lin - sample * H;
+        i0 = 0;
+        i1 = tiles;
+    } else {
+        const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H / HG, heads_magic);
+        sample = wi.sample;
+        head0 = wi.head * HG;
+        i0 = wi.strip * nt;
+        i1 = min(i0 + nt, tiles);
+    }
+    const uint32_t head = head0 + hw, b = sample * H + head;
     const int g = lane >> 4, n = lane & 15;
 
     // resources end with the strip (plus its halo), so the fixed-size copy below
     // fetches nothing beyond what this strip needs
-    const int64_t in_off = sample * in.sample + head0 * in.head, out_off = sample * outl.sample + head * outl.head;
-    const int key_bytes = min(T, 16 * (i1 + 1)) * in.pitch, qry_bytes = min(T, 16 * i1) * in.pitch;
+    // first what the strip copies need, and nothing else: a workgroup's life starts with the time to its first copy
+    const int64_t in_off = sample * in.sample + head0 * in.head;
+    const int key_bytes = (ONE ? T : min(T, 16 * (i1 + 1))) * in.pitch, qry_bytes = (ONE ? T : min(T, 16 * i1)) * in.pitch;
     const Rsrc qs = make_rsrc(q + in_off, qry_bytes), ks = make_rsrc(k + in_off, key_bytes);
-    const Rsrc vs = make_rsrc(v + in_off, key_bytes), os = make_rsrc(out + out_off, T * outl.pitch);
-    const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
-    const bool out_whole_lines = stores_whole_lines(outl.pitch, C, 0);
-    const bool out_grouped = HG > 1 && outl.head == 2 * C && outl.width == 2 * C && outl.pitch >= HG * 2 * C;
-
-    BiasTable bias_raw;
-    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
+    const Rsrc vs = make_rsrc(v + in_off, key_bytes);
 
     // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
     constexpr int TW = NW / HG;                      // tiles the workgroup computes side by side
@@ -79,13 +94,21 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
         };
         using Once = std::integral_constant<int, kReadOnce>;
         using Shared = std::integral_constant<int, kReadShared>;
-        if (strips == 1 && whole_lines)         // nobody else reads these rows' lines
+        if ((ONE || strips == 1) && whole_lines)         // nobody else reads these rows' lines
             stage(Once{}, Once{});
-        else if (whole_lines)
+        else if (!ONE && whole_lines)
             stage(Shared{}, Once{});
         else
             stage(Shared{}, Shared{});
     }
+    __builtin_amdgcn_sched_barrier(0);       // the copies are on their way: everything else is worked out behind them
+    BiasTable bias_raw;                      // (the wait for the copies covers this load too, wherever it is issued)
+    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
+    const int64_t out_off = sample * outl.sample + head * outl.head;
+    const Rsrc os = make_rsrc(out + out_off, T * outl.pitch);
+    const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
+    const bool out_whole_lines = stores_whole_lines(outl.pitch, C, 0);
+    const bool out_grouped = HG > 1 && outl.head == 2 * C && outl.width == 2 * C && outl.pitch >= HG * 2 * C;
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, load_uniform_i32(t_valid, sample)));
@@ -266,13 +289,18 @@ int launch_fwd_hg(void *out, float *lse, const void *q, const void *k, const voi
     const Split sp = make_split(g.B / HG, g.T, HG > 1 ? kGroupTiles : Strip<C>::kMaxTiles);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
     const bool two = window_blocks(g) == 2;
+    constexpr bool kCanOne = HG == 1;
+    const bool one = kCanOne && sp.strips == 1;
     auto kern = g.drop.threshold
-                    ? (two ? fused_fwd_kernel<DT, C, 2, true, HG> : fused_fwd_kernel<DT, C, 3, true, HG>)
-                    : (two ? fused_fwd_kernel<DT, C, 2, false, HG> : fused_fwd_kernel<DT, C, 3, false, HG>);
+                    ? (two ? (one ? fused_fwd_kernel<DT, C, 2, true, HG, kCanOne> : fused_fwd_kernel<DT, C, 2, true, HG, false>)
+                           : (one ? fused_fwd_kernel<DT, C, 3, true, HG, kCanOne> : fused_fwd_kernel<DT, C, 3, true, HG, false>))
+                    : (two ? (one ? fused_fwd_kernel<DT, C, 2, false, HG, kCanOne> : fused_fwd_kernel<DT, C, 2, false, HG, false>)
+                           : (one ? fused_fwd_kernel<DT, C, 3, false, HG, kCanOne> : fused_fwd_kernel<DT, C, 3, false, HG, false>));
     const size_t lds = (size_t)2 * region_bytes<C * HG>(sp.nt + 2) + region_bytes<C * HG>(sp.nt) +
                        HG * kBiasEntries * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
-    note_kernel("fused_fwd_kernel", DT::tag, C, two ? 2 : 3, g.drop.threshold != 0, HG);
+    note_kernel_as("fused_fwd_kernel<%s, %d, %d, %s, %d, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C, two ? 2 : 3,
+                   g.drop.threshold ? "true" : "false", HG, one ? "true" : "false");
     launch_kernel_block(kern, (unsigned)sp.items, 64u * (HG > 1 ? kGroupWaves : kWaves), lds, s, (char *)out, lse,
                   (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
@@ -378,17 +406,29 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // the head's bias table, read before pass 1 only: in what the score tiles need beyond the K and V regions, if that is room enough
     LDS_PTR(float) bias_lds = bwd_bias_in_padding(kv_bytes, key_region) ? (LDS_PTR(float))(k_lds + 2 * key_region) : lse_lds + kLseRows;
     LDS_PTR(float) rsum = lse_lds;                                          // [kWaves][32] d rpb slot sums per wave, once every wave has read its lse
-    const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
-    const uint32_t item = wi.item, b = wi.sample * H + wi.head, sample = wi.sample, head = wi.head;
-    const int i0 = wi.strip * nt, i1 = min(i0 + nt, tiles);
+    uint32_t item, sample, head;
+    int i0, i1;
+    if constexpr (ONE) {              // as in the forward: no strips; packed rows have no neighbours to share an L2 with
+        item = in.pitch == 2 * C && outl.pitch == 2 * C ? blockIdx.x : xcd_item(blockIdx.x, items);
+        sample = div_by(item, H, heads_magic);
+        head = item - sample * H;
+        i0 = 0;
+        i1 = tiles;
+    } else {
+        const WorkItem wi = work_item(blockIdx.x, items, strips, strips_magic, H, heads_magic);
+        item = wi.item;
+        sample = wi.sample;
+        head = wi.head;
+        i0 = wi.strip * nt;
+        i1 = min(i0 + nt, tiles);
+    }
+    const uint32_t b = sample * H + head;
     const int g = lane >> 4, n = lane & 15;
 
     const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
-    BiasTable bias_raw;
-    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
     {
-        const int key_bytes = min(T, 16 * (i1 + 2)) * in.pitch;
-        const int qry_rows = min(T, 16 * (i1 + HALO));
+        const int key_bytes = (ONE ? T : min(T, 16 * (i1 + 2))) * in.pitch;
+        const int qry_rows = ONE ? T : min(T, 16 * (i1 + HALO));
         const Rsrc ks = make_rsrc(k + in_off, key_bytes), vs = make_rsrc(v + in_off, key_bytes);
         const Rsrc qs = make_rsrc(q + in_off, qry_rows * in.pitch), gs = make_rsrc(dout + out_off, qry_rows * outl.pitch);
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
@@ -408,6 +448,9 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
             stage_direct<C, MT + 2 * HALO, kReadShared>(gs, 16 * (i0 - HALO), g_lds, nt + 2 * HALO, wave, lane_off_g, outl.pitch);
         }
     }
+    __builtin_amdgcn_sched_barrier(0);       // the copies are on their way: everything else is worked out behind them
+    BiasTable bias_raw;                      // (the wait for the copies covers this load too, wherever it is issued)
+    load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
 
     int tv = T;
     if (t_valid) tv = max(0, min(T, load_uniform_i32(t_valid, sample)));

@@ -147,8 +147,8 @@ template <int C> struct Strip {
 // workgroup barrier that publishes the regions.
 constexpr int kChunk = 1024;
 static_assert(kWaves % 4 == 0, "chunk -> swizzle phase mapping assumes a multiple of four waves");
-template <int C> constexpr int region_bytes(int ntiles) {
-    return (ntiles * Lds<C>::kTileBytes + kChunk - 1) / kChunk * kChunk;
+template <int C> constexpr int region_bytes(int ntiles) {      // unsigned: a shift and a mask where the count is a run-time value
+    return (int)(((uint32_t)(ntiles * Lds<C>::kTileBytes) + kChunk - 1) / kChunk * kChunk);
 }
 // `pitch` is the distance in bytes between consecutive rows in memory, `width` the bytes of a row that exist
 // there (2 * head_dim; both 2*C when the rows are packed and as wide as the kernel's C).  A head_dim below C is
@@ -185,7 +185,7 @@ __device__ inline void stage_direct(Rsrc src, int row_lo, LDS_PTR(char) region, 
     static_assert(NW % 4 == 0, "chunk -> swizzle phase mapping assumes a multiple of four waves");
     constexpr int kRounds = (region_bytes<C>(NTILES) / kChunk + NW - 1) / NW;
     constexpr int kChunkRows = kChunk / Lds<C>::kRowBytes;
-    const int chunks = region_bytes<C>(ntiles) / kChunk;
+    const int chunks = (int)((uint32_t)region_bytes<C>(ntiles) / kChunk);
     const int base = row_lo * pitch + lane_off, step = kChunkRows * pitch;
 #pragma unroll
     for (int j = 0; j < kRounds; ++j) {
@@ -391,7 +391,7 @@ struct BiasTable {
 // wait_bias() behind any wait that covers the loads issued up to here (loads return in the order they were issued).
 __device__ inline void load_bias_table(BiasTable &t, const float *rpb_h, int W, int lane) {
     const uint64_t p = reinterpret_cast<uint64_t>(rpb_h);
-    const u32x4 rs = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, rpb_h ? (uint32_t)W * 4u : 0u, 0x00020000u};   // NULL: empty, reads as zeros
+    const u32x4 rs = {(uint32_t)p, (uint32_t)(p >> 32) & 0xffffu, p ? (uint32_t)W * 4u : 0u, 0x00020000u};   // NULL: empty, reads as zeros
     const int off = (lane - kBiasPad) * 4;                                                                         // outside [0, W): 0
     asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "=v"(t.raw) : "v"(off), "s"(rs) : "memory");
 }
