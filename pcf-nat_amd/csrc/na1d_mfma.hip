@@ -22,7 +22,9 @@ constexpr int kGroupWaves = 8;               // waves per workgroup when heads a
 // then, and what a workgroup works out before its first copy can go - strip arithmetic, the XCD-aware order - is cut to
 // the sample / head split and three buffer resources: at T around 100 a launch is one round of workgroups, and every
 // instruction in front of the first copy is in the launch's duration (6 ns apiece, measured by adding some).
-template <class DT, int C, int NBV, bool DROP, int HG, bool ONE>
+// ONE == 2: such strips of packed rows as wide as the kernel's C (pitch = width = 2*C bytes, in and out): pitch, LDS
+// layout (regions for the most tiles a strip can have) and the copies' chunk counts become constants as well.
+template <class DT, int C, int NBV, bool DROP, int HG, int ONE>
 __global__ void __launch_bounds__(64 * (HG > 1 ? kGroupWaves : kWaves))
 fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const float *__restrict__ rpb,
@@ -37,6 +39,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     constexpr int MT = HG > 1 ? kGroupTiles : Strip<CS>::kMaxTiles;
     static_assert(NW % HG == 0, "whole waves per head");
     static_assert(!ONE || HG == 1, "the whole-sequence form is for single heads");
+    constexpr bool PK = ONE == 2;
     fetch_args_now(out, lse, q, k, v, rpb, t_valid, items, T, W, L, H, tiles, nt, strips, scale, strips_magic, heads_magic,
                    in.sample, in.head, in.pitch, in.width, outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
@@ -44,18 +47,24 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     // copies that start on a tile boundary measured faster here than ones that start at the first key, and the
     // forward is not short of LDS), Q region of nt tiles
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int key_region = region_bytes<CS>(nt + 2);
+    const int key_region = region_bytes<CS>(PK ? MT + 2 : nt + 2);
     LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + key_region;
     LDS_PTR(char) q_lds = v_lds + key_region;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + region_bytes<CS>(nt)) + (HG > 1 ? wave % HG : 0) * kBiasEntries;   // the bias table of this wave's head
+    LDS_PTR(float) bias_lds = (LDS_PTR(float))(q_lds + region_bytes<CS>(PK ? MT : nt)) + (HG > 1 ? wave % HG : 0) * kBiasEntries;   // the bias table of this wave's head
     const int hw = HG > 1 ? wave % HG : 0;           // this wave's head inside the group
-    uint32_t sample, head0;
+    uint32_t sample, head0, lin_pk = 0;
     int i0, i1;
-    if constexpr (ONE) {
+    if constexpr (PK) {
+        lin_pk = blockIdx.x;
+        sample = div_by(lin_pk, H, heads_magic);
+        head0 = lin_pk - sample * H;
+        i0 = 0;
+        i1 = tiles;
+    } else if constexpr (ONE != 0) {
         // heads that interleave in memory share lines: their workgroups stay on one XCD, behind one L2 (xcd_item);
         // packed rows are nobody else's, and the plain order is 3 % faster
         const uint32_t lin = in.pitch == 2 * C && outl.pitch == 2 * C ? blockIdx.x : xcd_item(blockIdx.x, items);
@@ -76,14 +85,20 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     // resources end with the strip (plus its halo), so the fixed-size copy below
     // fetches nothing beyond what this strip needs
     // first what the strip copies need, and nothing else: a workgroup's life starts with the time to its first copy
-    const int64_t in_off = sample * in.sample + head0 * in.head;
-    const int key_bytes = (ONE ? T : min(T, 16 * (i1 + 1))) * in.pitch, qry_bytes = (ONE ? T : min(T, 16 * i1)) * in.pitch;
+    const int in_pitch = PK ? 2 * C : in.pitch;
+    const int64_t in_off = PK ? (int64_t)((uint64_t)lin_pk * (uint32_t)(T * 2 * C)) : sample * in.sample + head0 * in.head;
+    const int key_bytes = (ONE ? T : min(T, 16 * (i1 + 1))) * in_pitch, qry_bytes = (ONE ? T : min(T, 16 * i1)) * in_pitch;
     const Rsrc qs = make_rsrc(q + in_off, qry_bytes), ks = make_rsrc(k + in_off, key_bytes);
     const Rsrc vs = make_rsrc(v + in_off, key_bytes);
 
     // stage the strip: K and V rows [16*i0 - 16, 16*i0 + 16*(MT+1)), Q rows [16*i0, 16*i0 + 16*MT)
     constexpr int TW = NW / HG;                      // tiles the workgroup computes side by side
-    {
+    if constexpr (PK) {
+        const int lane_off = direct_lane_offset<CS>(wave, lane);
+        stage_packed<CS, MT + 2, kReadOnce, NW>(ks, -16, k_lds, wave, lane_off);
+        stage_packed<CS, MT, kReadOnce, NW>(qs, 0, q_lds, wave, lane_off);
+        stage_packed<CS, MT + 2, kReadOnce, NW>(vs, -16, v_lds, wave, lane_off);
+    } else {
         const int lane_off = direct_lane_offset<CS>(wave, lane, in.pitch, HG * in.width);
         const bool whole_lines = in.pitch == 2 * C || CS % 64 == 0;
         auto stage = [&](auto key_aux, auto qry_aux) {
@@ -104,10 +119,11 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
     __builtin_amdgcn_sched_barrier(0);       // the copies are on their way: everything else is worked out behind them
     BiasTable bias_raw;                      // (the wait for the copies covers this load too, wherever it is issued)
     load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
-    const int64_t out_off = sample * outl.sample + head * outl.head;
-    const Rsrc os = make_rsrc(out + out_off, T * outl.pitch);
+    const int out_pitch = PK ? 2 * C : outl.pitch, out_width = PK ? 2 * C : outl.width;
+    const int64_t out_off = PK ? in_off : sample * outl.sample + head * outl.head;
+    const Rsrc os = make_rsrc(out + out_off, T * out_pitch);
     const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
-    const bool out_whole_lines = stores_whole_lines(outl.pitch, C, 0);
+    const bool out_whole_lines = stores_whole_lines(out_pitch, C, 0);
     const bool out_grouped = HG > 1 && outl.head == 2 * C && outl.width == 2 * C && outl.pitch >= HG * 2 * C;
 
     int tv = T;
@@ -249,7 +265,7 @@ fused_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__
             for (int ct = 0; ct < CT; ++ct)
                 *reinterpret_cast<LDS_PTR(u32x2)>(q_mine + tile_bytes + LL::addr(n, hw * 2 * C + 32 * ct + 8 * g)) = ow[ct];
         } else {
-            store_tile<C>(os, qrow * outl.pitch, ow, g, out_whole_lines, outl.width);
+            store_tile<C>(os, qrow * out_pitch, ow, g, out_whole_lines, out_width);
         }
         if (lse && g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(lse_row), ls, qrow * 4, 0, 0);
     }
@@ -289,18 +305,29 @@ int launch_fwd_hg(void *out, float *lse, const void *q, const void *k, const voi
     const Split sp = make_split(g.B / HG, g.T, HG > 1 ? kGroupTiles : Strip<C>::kMaxTiles);
     if (!items_ok(sp, g) || !strides_ok(in, g) || !strides_ok(outl, g)) return NA1D_ERR_UNSUPPORTED;
     const bool two = window_blocks(g) == 2;
-    constexpr bool kCanOne = HG == 1;
-    const bool one = kCanOne && sp.strips == 1;
-    auto kern = g.drop.threshold
-                    ? (two ? (one ? fused_fwd_kernel<DT, C, 2, true, HG, kCanOne> : fused_fwd_kernel<DT, C, 2, true, HG, false>)
-                           : (one ? fused_fwd_kernel<DT, C, 3, true, HG, kCanOne> : fused_fwd_kernel<DT, C, 3, true, HG, false>))
-                    : (two ? (one ? fused_fwd_kernel<DT, C, 2, false, HG, kCanOne> : fused_fwd_kernel<DT, C, 2, false, HG, false>)
-                           : (one ? fused_fwd_kernel<DT, C, 3, false, HG, kCanOne> : fused_fwd_kernel<DT, C, 3, false, HG, false>));
-    const size_t lds = (size_t)2 * region_bytes<C * HG>(sp.nt + 2) + region_bytes<C * HG>(sp.nt) +
-                       HG * kBiasEntries * sizeof(float);
+    // the kernel's form: 0 strips of longer sequences or grouped heads, 1 whole sequences, 2 whole sequences of packed
+    // 16-channel rows (where regions for the longest strip cost no workgroup: the forward is not short of LDS there)
+    constexpr int kOne = HG == 1 ? 1 : 0, kPacked = HG == 1 && C == 16 ? 2 : kOne;
+    const Strides ib = byte_strides(in, g), ob = byte_strides(outl, g);
+    auto packed = [&](const Strides &x) {           // [B, T, C] with nothing between rows, heads or samples
+        return x.pitch == 2 * C && x.width == 2 * C && x.head == g.T * 2 * C && x.sample == (int64_t)g.H * g.T * 2 * C;
+    };
+    const int one = HG > 1 || sp.strips != 1 ? 0 : (kPacked == 2 && packed(ib) && packed(ob) && g.T * 2 * C < (1 << 30)) ? 2 : 1;
+    auto pick = [&](auto nbv, auto drop) {
+        constexpr int N = decltype(nbv)::value;
+        constexpr bool D = decltype(drop)::value;
+        return one == 2 ? fused_fwd_kernel<DT, C, N, D, HG, kPacked> : one == 1 ? fused_fwd_kernel<DT, C, N, D, HG, kOne>
+                                                                                 : fused_fwd_kernel<DT, C, N, D, HG, 0>;
+    };
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    auto kern = g.drop.threshold ? (two ? pick(I2{}, std::true_type{}) : pick(I3{}, std::true_type{}))
+                                 : (two ? pick(I2{}, std::false_type{}) : pick(I3{}, std::false_type{}));
+    const int lt = one == 2 ? Strip<C>::kMaxTiles : sp.nt;          // tiles the regions are laid out for
+    const size_t lds = (size_t)2 * region_bytes<C * HG>(lt + 2) + region_bytes<C * HG>(lt) + HG * kBiasEntries * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     note_kernel_as("fused_fwd_kernel<%s, %d, %d, %s, %d, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C, two ? 2 : 3,
-                   g.drop.threshold ? "true" : "false", HG, one ? "true" : "false");
+                   g.drop.threshold ? "true" : "false", HG, one == 2 ? "2" : one == 1 ? "1" : "0");
     launch_kernel_block(kern, (unsigned)sp.items, 64u * (HG > 1 ? kGroupWaves : kWaves), lds, s, (char *)out, lse,
                   (const char *)q, (const char *)k, (const char *)v,
                   rpb, t_valid, (uint32_t)sp.items, (int)g.T, g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale,
@@ -366,8 +393,10 @@ template <int C> constexpr int bwd_lse_rows(bool one) {
 // ONE: the strip is the whole sequence (strips == 1).  There are no neighbouring strips then and no halo tiles of
 // queries either side: two tiles fewer in the Q and dO regions and in a wave's share of pass 1, which is what lets a
 // seventh workgroup of 16-channel heads onto a CU (LDS and registers both).
-template <class DT, int C, int NBV, bool DROP, bool ONE>
-__global__ void __launch_bounds__(kThreads, bwd_min_waves(C, DROP, ONE))
+// ONE == 2: such a strip of packed rows as wide as the kernel's C, in and out: the pitch is a constant, the rows of work
+// item i start i * T * 2C bytes into every tensor, and the sample / head split waits until the copies are on their way.
+template <class DT, int C, int NBV, bool DROP, int ONE>
+__global__ void __launch_bounds__(kThreads, bwd_min_waves(C, DROP, ONE != 0))
 fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, float *__restrict__ drpb,
                  const char *__restrict__ q, const char *__restrict__ k, const char *__restrict__ v,
                  const char *__restrict__ dout, const float *__restrict__ lse, const float *__restrict__ rpb,
@@ -382,11 +411,12 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                    drpb_partial, kv_bytes, strips_magic, heads_magic, in.sample, in.head, in.pitch, in.width,
                    outl.sample, outl.head, outl.pitch, outl.width, shift_arg);
     if constexpr (DROP) fetch_args_now(drop.threshold, drop.seed_lo, drop.seed_hi, drop.inv_keep, drop.row_stride, drop.row_offset, drop.seq_rows);
+    constexpr bool PK = ONE == 2;
     constexpr int HALO = ONE ? 0 : 1;                      // query tiles either side of the strip whose scores pass 2 needs
     constexpr int kRowsQ = (MT + 2 * HALO) * 16;
     constexpr int TPW = (MT + 2 * HALO + kWaves - 1) / kWaves;    // query tiles per wave, at most
     constexpr int kScoreTile = 16 * 16 * 2;                // one 16x16 tile of 16-bit scores
-    constexpr int kLseRows = bwd_lse_rows<C>(ONE);
+    constexpr int kLseRows = bwd_lse_rows<C>(ONE != 0);
     static_assert(kRowsQ <= kLseRows && kLseRows <= kThreads, "one lane per staged lse row");
     // dynamic LDS (see launch_bwd): [K region | V region] of nt+1+NBV tiles each, starting at the first key of
     // query tile i0-1 (row 16*(i0-1) - shift, so that virtual key blocks are whole tiles of the region), reused after
@@ -406,9 +436,13 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     // the head's bias table, read before pass 1 only: in what the score tiles need beyond the K and V regions, if that is room enough
     LDS_PTR(float) bias_lds = bwd_bias_in_padding(kv_bytes, key_region) ? (LDS_PTR(float))(k_lds + 2 * key_region) : lse_lds + kLseRows;
     LDS_PTR(float) rsum = lse_lds;                                          // [kWaves][32] d rpb slot sums per wave, once every wave has read its lse
-    uint32_t item, sample, head;
+    uint32_t item, sample = 0, head = 0;
     int i0, i1;
-    if constexpr (ONE) {              // as in the forward: no strips; packed rows have no neighbours to share an L2 with
+    if constexpr (PK) {
+        item = blockIdx.x;
+        i0 = 0;
+        i1 = tiles;
+    } else if constexpr (ONE != 0) {   // as in the forward: no strips; packed rows have no neighbours to share an L2 with
         item = in.pitch == 2 * C && outl.pitch == 2 * C ? blockIdx.x : xcd_item(blockIdx.x, items);
         sample = div_by(item, H, heads_magic);
         head = item - sample * H;
@@ -422,21 +456,29 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         i0 = wi.strip * nt;
         i1 = min(i0 + nt, tiles);
     }
-    const uint32_t b = sample * H + head;
+    const uint32_t b = ONE ? item : sample * H + head;       // one strip per sequence: the item is the sequence
     const int g = lane >> 4, n = lane & 15;
 
-    const int64_t in_off = sample * in.sample + head * in.head, out_off = sample * outl.sample + head * outl.head;
+    const int in_pitch = PK ? 2 * C : in.pitch, out_pitch = PK ? 2 * C : outl.pitch;
+    const int in_width = PK ? 2 * C : in.width;
+    const int64_t in_off = PK ? (int64_t)((uint64_t)item * (uint32_t)(T * 2 * C)) : sample * in.sample + head * in.head;
+    const int64_t out_off = PK ? in_off : sample * outl.sample + head * outl.head;
     {
-        const int key_bytes = (ONE ? T : min(T, 16 * (i1 + 2))) * in.pitch;
+        const int key_bytes = (ONE ? T : min(T, 16 * (i1 + 2))) * in_pitch;
         const int qry_rows = ONE ? T : min(T, 16 * (i1 + HALO));
         const Rsrc ks = make_rsrc(k + in_off, key_bytes), vs = make_rsrc(v + in_off, key_bytes);
-        const Rsrc qs = make_rsrc(q + in_off, qry_rows * in.pitch), gs = make_rsrc(dout + out_off, qry_rows * outl.pitch);
+        const Rsrc qs = make_rsrc(q + in_off, qry_rows * in_pitch), gs = make_rsrc(dout + out_off, qry_rows * out_pitch);
         const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4);
-        const int lane_off = direct_lane_offset<C>(wave, lane, in.pitch, in.width);
-        const int lane_off_g = direct_lane_offset<C>(wave, lane, outl.pitch, outl.width);
+        const int lane_off = PK ? direct_lane_offset<C>(wave, lane) : direct_lane_offset<C>(wave, lane, in.pitch, in.width);
+        const int lane_off_g = PK ? lane_off : direct_lane_offset<C>(wave, lane, outl.pitch, outl.width);
         // lse of the query-side rows, one per lane (natural log; rows past the region's end are never read)
         if (64 * wave < kRowsQ) load_to_lds<4, 0>(ls, (LDS_PTR(char))(lse_lds + 64 * wave), (16 * (i0 - HALO) + tid) * 4);
-        if (ONE && (in.pitch == 2 * C || C % 64 == 0) && (outl.pitch == 2 * C || C % 64 == 0)) {
+        if constexpr (PK) {           // the pitch is the default argument, a constant
+            stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(ks, -16 - shift, k_lds, nt + 1 + NBV, wave, lane_off);
+            stage_direct<C, MT, kReadOnceBwd>(qs, 0, q_lds, nt, wave, lane_off);
+            stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(vs, -16 - shift, v_lds, nt + 1 + NBV, wave, lane_off);
+            stage_direct<C, MT, kReadOnceBwd>(gs, 0, g_lds, nt, wave, lane_off);
+        } else if (ONE && (in.pitch == 2 * C || C % 64 == 0) && (outl.pitch == 2 * C || C % 64 == 0)) {
             stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(ks, 16 * i0 - 16 - shift, k_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
             stage_direct<C, MT + 2 * HALO, kReadOnceBwd>(qs, 16 * (i0 - HALO), q_lds, nt + 2 * HALO, wave, lane_off, in.pitch);
             stage_direct<C, MT + 1 + NBV, kReadOnceBwd>(vs, 16 * i0 - 16 - shift, v_lds, nt + 1 + NBV, wave, lane_off, in.pitch);
@@ -449,6 +491,10 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         }
     }
     __builtin_amdgcn_sched_barrier(0);       // the copies are on their way: everything else is worked out behind them
+    if constexpr (PK) {
+        sample = div_by(item, H, heads_magic);
+        head = item - sample * H;
+    }
     BiasTable bias_raw;                      // (the wait for the copies covers this load too, wherever it is issued)
     load_bias_table(bias_raw, rpb ? rpb + head * W : nullptr, W, lane);
 
@@ -490,8 +536,8 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
 
     // ---------------- pass 1: query tiles i0-HALO .. i1-1+HALO -> dQ, d rpb, score tiles ----------------
     float racc_x[4] = {0.f, 0.f, 0.f, 0.f}, racc_y[4] = {0.f, 0.f, 0.f, 0.f};
-    const Rsrc dqs = make_rsrc(dq + in_off, T * in.pitch);
-    const bool dq_whole_lines = stores_whole_lines(in.pitch, C, 0);
+    const Rsrc dqs = make_rsrc(dq + in_off, T * in_pitch);
+    const bool dq_whole_lines = stores_whole_lines(in_pitch, C, 0);
     u32x2 sc[TPW][2][2];                // [tile of this wave][X/Y slot set][P / dS], rounded to 16 bit
 #pragma unroll
     for (int jt = 0; jt < TPW; ++jt) {
@@ -595,7 +641,7 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
         u32x2 qw[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[ct], scale);
-        store_tile<C>(dqs, qrow * in.pitch, qw, g, dq_whole_lines, in.width);
+        store_tile<C>(dqs, qrow * in_pitch, qw, g, dq_whole_lines, in_width);
     }
 
     // d rpb: the window slot of each of a lane's 8 score registers is the same for every tile, so the lane
@@ -652,12 +698,12 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
     }
     const int sc_lane = (4 * g + (n >> 2)) * 32 + (n & 3) * 8;       // transposed read of a score tile
     const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
-    const Rsrc dks = make_rsrc(dk + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
-    const Rsrc dvs = make_rsrc(dv + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
+    const Rsrc dks = make_rsrc(dk + in_off + (int64_t)row_lo * in_pitch, (row_hi - row_lo) * in_pitch);
+    const Rsrc dvs = make_rsrc(dv + in_off + (int64_t)row_lo * in_pitch, (row_hi - row_lo) * in_pitch);
     const int kp_lo = i0 + (shift == 16 ? 1 : 0), kp_hi = i1 - (shift == 0 ? 1 : 0);
     // a key block starts `shift` rows before a tile (non-temporal stores of split lines cost cfg2's backward 5 %;
     // where lines are whole they gain 10 %)
-    const bool whole_lines = stores_whole_lines(in.pitch, C, shift);
+    const bool whole_lines = stores_whole_lines(in_pitch, C, shift);
     for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
         f32x4 acck[CT], accv[CT];
 #pragma unroll
@@ -689,15 +735,15 @@ fused_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict_
                 acck[ct] = Mma<DT>::k16(read_tr(qtile + qry_tr.off[ct]), db, acck[ct]);
             }
         }
-        const int row_off = (16 * (kp - i0) - shift + n) * in.pitch;    // outside the strip -> dropped
+        const int row_off = (16 * (kp - i0) - shift + n) * in_pitch;    // outside the strip -> dropped
         u32x2 kw[CT], vw[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             kw[ct] = pack_acc<DT>(acck[ct], scale);
             vw[ct] = pack_acc<DT>(accv[ct], 1.f);
         }
-        store_tile<C>(dks, row_off, kw, g, whole_lines, in.width);
-        store_tile<C>(dvs, row_off, vw, g, whole_lines, in.width);
+        store_tile<C>(dks, row_off, kw, g, whole_lines, in_width);
+        store_tile<C>(dvs, row_off, vw, g, whole_lines, in_width);
     }
 
     // last, behind the gradient stores: issued earlier (the sums are complete before pass 2) the atomics cost the
@@ -729,11 +775,20 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
     }
     const bool two = window_blocks(g) == 2;
     const bool one = sp.strips == 1;
-    auto kern = g.drop.threshold
-                    ? (two ? (one ? fused_bwd_kernel<DT, C, 2, true, true> : fused_bwd_kernel<DT, C, 2, true, false>)
-                           : (one ? fused_bwd_kernel<DT, C, 3, true, true> : fused_bwd_kernel<DT, C, 3, true, false>))
-                    : (two ? (one ? fused_bwd_kernel<DT, C, 2, false, true> : fused_bwd_kernel<DT, C, 2, false, false>)
-                           : (one ? fused_bwd_kernel<DT, C, 3, false, true> : fused_bwd_kernel<DT, C, 3, false, false>));
+    const Strides ib = byte_strides(in, g), ob = byte_strides(outl, g);
+    auto packed = [&](const Strides &x) {           // [B, T, C] with nothing between rows, heads or samples
+        return x.pitch == 2 * C && x.width == 2 * C && x.head == g.T * 2 * C && x.sample == (int64_t)g.H * g.T * 2 * C;
+    };
+    const int form = !one ? 0 : packed(ib) && packed(ob) && g.T * 2 * C < (1 << 30) ? 2 : 1;      // see the kernel's ONE
+    auto pick = [&](auto nbv, auto drop) {
+        constexpr int N = decltype(nbv)::value;
+        constexpr bool D = decltype(drop)::value;
+        return form == 2 ? fused_bwd_kernel<DT, C, N, D, 2> : form == 1 ? fused_bwd_kernel<DT, C, N, D, 1> : fused_bwd_kernel<DT, C, N, D, 0>;
+    };
+    using I2 = std::integral_constant<int, 2>;
+    using I3 = std::integral_constant<int, 3>;
+    auto kern = g.drop.threshold ? (two ? pick(I2{}, std::true_type{}) : pick(I3{}, std::true_type{}))
+                                 : (two ? pick(I2{}, std::false_type{}) : pick(I3{}, std::false_type{}));
     // the K and V regions double as the score tiles of pass 2 (4 tiles of 512 B per query tile)
     // (a strip that is the whole sequence has no halo tiles)
     const int halo = one ? 0 : 1;
@@ -743,11 +798,11 @@ int launch_bwd(void *dq, void *dk, void *dv, float *drpb, const void *q, const v
                        (bwd_lse_rows<C>(one) + (bias_apart ? kBiasEntries : 0)) * sizeof(float);
     if (!allow_lds(kern, lds)) return NA1D_ERR_LAUNCH;
     note_kernel_as("fused_bwd_kernel<%s, %d, %d, %s, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C, two ? 2 : 3,
-                   g.drop.threshold ? "true" : "false", one ? "true" : "false");
+                   g.drop.threshold ? "true" : "false", form == 2 ? "2" : form == 1 ? "1" : "0");
     launch_kernel(kern, (unsigned)sp.items, lds, s, (char *)dq, (char *)dk, (char *)dv, drpb, (const char *)q,
                   (const char *)k, (const char *)v, (const char *)dout, lse, rpb, t_valid, (uint32_t)sp.items, (int)g.T,
                   g.W, g.L, g.H, sp.tiles, sp.nt, sp.strips, scale, partial, kv_bytes, div_magic(sp.strips),
-                  div_magic(g.H), byte_strides(in, g), byte_strides(outl, g), window_shift(g), g.drop);
+                  div_magic(g.H), ib, ob, window_shift(g), g.drop);
     // not behind a launch that was refused (events set on a capturing stream): the sums it would fold do not exist
     if (partial && drpb && !launch_events().refused)
         drpb_reduce_kernel<kPartialStride><<<(unsigned)(g.H * g.W), 128, 0, s>>>(drpb, partial, (int)(g.B / g.H), g.H, sp.strips, g.W);

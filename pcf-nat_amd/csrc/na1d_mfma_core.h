@@ -210,6 +210,19 @@ __device__ inline void stage_exact(Rsrc src, LDS_PTR(char) region, int bytes, in
         }
     }
 }
+// The same for packed rows (pitch = width = 2*C bytes) into a region of NTILES tiles, all of it: how many chunks there
+// are, which of them a wave loads and where they go is then known at compile time, and a copy is an add for M0 and the
+// load (rows past the resource's end are asked for all the same; they cost an instruction, no traffic).
+template <int C, int NTILES, int AUX, int NW = kWaves>
+__device__ inline void stage_packed(Rsrc src, int row_lo, LDS_PTR(char) region, int wave, int lane_off) {
+    static_assert(NW % 4 == 0, "chunk -> swizzle phase mapping assumes a multiple of four waves");
+    constexpr int kChunks = region_bytes<C>(NTILES) / kChunk, kRounds = (kChunks + NW - 1) / NW;
+    const int base = row_lo * Lds<C>::kRowBytes + lane_off + wave * kChunk;     // a chunk of packed rows is a chunk of memory
+    LDS_PTR(char) mine = region + wave * kChunk;
+#pragma unroll
+    for (int j = 0; j < kRounds; ++j)
+        if ((j + 1) * NW <= kChunks || wave < kChunks - j * NW) load_to_lds<16, AUX>(src, mine + j * NW * kChunk, base + j * NW * kChunk);
+}
 __device__ inline void wait_direct() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 // Workgroup barrier that waits for this wave's LDS accesses only.  __syncthreads() also waits for every vector-memory
 // access in flight, i.e. for strip copies that were issued early on purpose; what has to have landed is waited for
