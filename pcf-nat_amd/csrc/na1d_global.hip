@@ -68,9 +68,8 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     fetch_args_now(out, lse, q, k, v, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic, a.pitch, a.scale);
     if constexpr (DROP) fetch_args_now(a.drop.threshold, a.drop.seed_lo, a.drop.seed_hi, a.drop.inv_keep);
     constexpr int kStep = region_bytes<C>(kStripTiles);
-    extern __shared__ __attribute__((aligned(16))) char smem[];          // 3 * kStep bytes
-    LDS_PTR(char) q_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) k_lds = q_lds + kStep;
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 2 * kStep bytes
+    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
     LDS_PTR(char) v_lds = k_lds + kStep;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -99,20 +98,21 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     row_lane.init(0, lane);
     tr_lane.init(0, lane);
 
-    stage_direct<C, kStripTiles, kReadShared>(qs, 16 * kStripTiles * strip, q_lds, kStripTiles, wave, lane_off, a.pitch);
+    // the wave's query tile, which no other wave needs, straight into the registers of the matrix operand: a third less
+    // LDS, eight instead of six workgroups on a CU at 64 channels
+    RowOperand<C> qop;
+    load_rows<C, kReadShared>(qop, qs, 16 * qt * a.pitch, a.pitch, a.pitch, lane);
     float m = kNegInf, l = 0.f;
     f32x4 o[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-    RowOperand<C> qop;
 
     for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
-        if (c0) __syncthreads();                            // every wave is done with the previous chunk
+        if (c0) barrier_lds();                              // every wave is done with the previous chunk
         stage_direct<C, kStripTiles, kReadShared>(ks, 16 * c0, k_lds, kStripTiles, wave, lane_off, a.pitch);
         stage_direct<C, kStripTiles, kReadShared>(vs, 16 * c0, v_lds, kStripTiles, wave, lane_off, a.pitch);
         wait_direct();
-        __syncthreads();
-        if (c0 == 0) read_rows<C>(qop, q_lds + wave * LL::kTileBytes, row_lane);
+        barrier_lds();
         const int nk = min(kStripTiles, tiles - c0);        // key tiles in this chunk
         float z[kStripTiles][4];
         float mc = kNegInf;
@@ -170,6 +170,132 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
     store_tile<C>(os, qrow * a.pitch, ow, g, stores_whole_lines(a.pitch, C, 0), a.pitch);   // rows past T are dropped
     if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint((m + __builtin_amdgcn_logf(l)) * kLn2), ls, qrow * 4, 0, 0);
+}
+
+// =============================================================================
+// Forward for sequences of up to 128 rows (the models' dense layers run at about 100): one workgroup per sequence,
+// keys and values whole in LDS behind a single barrier, every wave two query tiles (wave and wave + 4) that share each
+// key and value operand it reads.  All scores of a row are in registers at once, so the softmax is a plain one.
+// =============================================================================
+constexpr int kShortTiles = 8;      // longest sequence of the short forms, in tiles
+template <class DT, int C, bool DROP, int TILES, int QT>
+__global__ void __launch_bounds__(64 * TILES / QT)
+global_fwd_short_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
+                        const char *__restrict__ k, const char *__restrict__ v, const int32_t *__restrict__ t_valid,
+                        GlobalArgs a) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16, kW = TILES / QT;       // waves of the workgroup, QT query tiles each
+    fetch_args_now(out, lse, q, k, v, t_valid, a.T, a.H, a.heads_magic, a.pitch, a.scale);
+    if constexpr (DROP) fetch_args_now(a.drop.threshold, a.drop.seed_lo, a.drop.seed_hi, a.drop.inv_keep);
+    const int T = a.T, tiles = (T + 15) >> 4, pitch = a.pitch;      // rows of head_dim channels, zero-padded to C on the way in
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 2 * region_bytes<C>(tiles)
+    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) v_lds = k_lds + region_bytes<C>(tiles);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, n = lane & 15;
+    const uint32_t b = blockIdx.x;
+    const int64_t seq_off = (int64_t)((uint64_t)b * (uint32_t)(T * pitch));
+    const Rsrc ks = make_rsrc(k + seq_off, T * pitch), vs = make_rsrc(v + seq_off, T * pitch);
+    const Rsrc qs = make_rsrc(q + seq_off, T * pitch);
+    const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
+    stage_direct<C, TILES, kReadOnce, kW>(ks, 0, k_lds, tiles, wave, lane_off, pitch);
+    stage_direct<C, TILES, kReadOnce, kW>(vs, 0, v_lds, tiles, wave, lane_off, pitch);
+    RowOperand<C> qop[QT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h) load_rows<C, kReadOnce>(qop[h], qs, 16 * (wave + kW * h) * pitch, pitch, pitch, lane);
+    __builtin_amdgcn_sched_barrier(0);
+
+    const uint32_t sample = div_by(b, a.H, a.heads_magic);
+    int tv = T;
+    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    const Rsrc os = make_rsrc(out + seq_off, T * pitch);
+    const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
+    const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
+    RowLane<C> row_lane;
+    TrLane<C> tr_lane;
+    row_lane.init(0, lane);
+    tr_lane.init(0, lane);
+    wait_direct();
+    barrier_lds();
+
+    float z[QT][TILES][4];
+#pragma unroll
+    for (int kt = 0; kt < TILES; ++kt) {
+        if (kt < tiles) {
+            RowOperand<C> kop;
+            read_rows<C>(kop, k_lds + kt * LL::kTileBytes, row_lane);
+#pragma unroll
+            for (int h = 0; h < QT; ++h) {
+                const bool row_masked = 16 * (wave + kW * h) + n >= tv;
+                const f32x4 s = dot_rows_mma<DT, C>(kop, qop[h]);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = 16 * kt + 4 * g + r;
+                    const float zz = s[r] * scale2 + ((key >= tv || row_masked) ? mask2 : 0.f);
+                    z[h][kt][r] = key < T ? zz : kNegInf;   // rows past the sequence do not exist
+                }
+            }
+        } else {
+#pragma unroll
+            for (int h = 0; h < QT; ++h)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) z[h][kt][r] = kNegInf;
+        }
+    }
+    u32x2 pb[QT][TILES];
+    float m[QT], l[QT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        const int qrow = 16 * (wave + kW * h) + n;
+        float mc = kNegInf;
+#pragma unroll
+        for (int kt = 0; kt < TILES; ++kt) mc = max3(mc, max2(z[h][kt][0], z[h][kt][1]), max2(z[h][kt][2], z[h][kt][3]));
+        m[h] = xor_max(mc);                                 // finite: key 0 exists
+        const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
+        float part = 0.f;
+#pragma unroll
+        for (int kt = 0; kt < TILES; ++kt) {
+            float p[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                p[r] = __builtin_amdgcn_exp2f(z[h][kt][r] - m[h]);
+                part += p[r];
+                // a dropped probability stays in the sum and leaves O
+                if (DROP && !dropout_keeps(drop_key, 16 * kt + 4 * g + r, a.drop)) p[r] = 0.f;
+            }
+            pb[h][kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+        }
+        l[h] = xor_sum(part);
+    }
+    f32x4 o[QT][CT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kt = 0; kt < TILES; ++kt) {
+        if (kt >= tiles) continue;
+        LDS_PTR(char) blk = v_lds + kt * LL::kTileBytes;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const auto vt = read_tr(blk + tr_lane.off[ct]);
+#pragma unroll
+            for (int h = 0; h < QT; ++h) o[h][ct] = Mma<DT>::k16(vt, pb[h][kt], o[h][ct]);
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        if (wave + kW * h >= tiles) break;
+        const int qrow = 16 * (wave + kW * h) + n;
+        const float inv = __builtin_amdgcn_rcpf(l[h]) * (DROP ? a.drop.inv_keep : 1.f);
+        u32x2 ow[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[h][ct], inv);
+        store_tile<C>(os, qrow * pitch, ow, g, stores_whole_lines(pitch, C, 0), pitch);     // rows past T are dropped
+        if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint((m[h] + __builtin_amdgcn_logf(l[h])) * kLn2), ls, qrow * 4, 0, 0);
+    }
 }
 
 // =============================================================================
@@ -392,6 +518,199 @@ global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__re
     store_tile<C>(dvs, key * a.pitch, vw, g, stream, a.pitch);
 }
 
+// =============================================================================
+// Backward for sequences of up to 128 rows: one workgroup per sequence and ONE kernel.  Q, K, V and dO sit whole in
+// LDS behind a single barrier.  Every wave first takes query tiles (delta and dQ, as global_dq_kernel), leaves delta
+// in LDS for the others, and then, behind a second barrier, key tiles (dK and dV, as global_dkv_kernel).  Each input
+// is read from memory once and delta never leaves the chip.
+// =============================================================================
+template <class DT, int C, bool DROP, int TILES, int QT>
+__global__ void __launch_bounds__(64 * TILES / QT)
+global_bwd_short_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__ dv, const char *__restrict__ q,
+                        const char *__restrict__ k, const char *__restrict__ v, const char *__restrict__ out,
+                        const char *__restrict__ dout, const float *__restrict__ lse, const int32_t *__restrict__ t_valid,
+                        GlobalArgs a) {
+    using LL = Lds<C>;
+    constexpr int CT = C / 16, kW = TILES / QT;       // waves of the workgroup, QT query / key tiles each
+    constexpr int kRows = 16 * TILES;
+    fetch_args_now(dq, dk, dv, q, k, v, out, dout, lse, t_valid, a.T, a.H, a.heads_magic, a.pitch, a.scale);
+    if constexpr (DROP) fetch_args_now(a.drop.threshold, a.drop.seed_lo, a.drop.seed_hi, a.drop.inv_keep);
+    const int T = a.T, tiles = (T + 15) >> 4, pitch = a.pitch;
+    const int region = region_bytes<C>(tiles);
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 4 * region + 2 * kRows * 4 bytes
+    LDS_PTR(char) q_lds = (LDS_PTR(char))smem;
+    LDS_PTR(char) g_lds = q_lds + region;                   // dO
+    LDS_PTR(char) k_lds = g_lds + region;
+    LDS_PTR(char) v_lds = k_lds + region;
+    LDS_PTR(float) lse_lds = (LDS_PTR(float))(v_lds + region);
+    LDS_PTR(float) del_lds = lse_lds + kRows;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 4, n = lane & 15;
+    const uint32_t b = blockIdx.x;
+    const int64_t seq_off = (int64_t)((uint64_t)b * (uint32_t)(T * pitch));
+    const Rsrc qs = make_rsrc(q + seq_off, T * pitch), gs = make_rsrc(dout + seq_off, T * pitch);
+    const Rsrc ks = make_rsrc(k + seq_off, T * pitch), vs = make_rsrc(v + seq_off, T * pitch);
+    const Rsrc os = make_rsrc(out + seq_off, T * pitch), ls = make_rsrc(lse + (int64_t)b * T, T * 4);
+    const int lane_off = direct_lane_offset<C>(wave, lane, pitch, pitch);
+    stage_direct<C, TILES, kReadOnce, kW>(qs, 0, q_lds, tiles, wave, lane_off, pitch);
+    stage_direct<C, TILES, kReadOnce, kW>(gs, 0, g_lds, tiles, wave, lane_off, pitch);
+    stage_direct<C, TILES, kReadOnce, kW>(ks, 0, k_lds, tiles, wave, lane_off, pitch);
+    stage_direct<C, TILES, kReadOnce, kW>(vs, 0, v_lds, tiles, wave, lane_off, pitch);
+    if (wave < kRows / 64) load_to_lds<4, 0>(ls, (LDS_PTR(char))(lse_lds + 64 * wave), (64 * wave + lane) * 4);     // rows past T: zeros
+    // this wave's own tiles (as queries first, as keys later); one past the sequence's last computes on that one and stores nothing
+    int own[QT];
+    RowOperand<C> oop[QT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        own[h] = min(wave + kW * h, tiles - 1);
+        load_rows<C, kReadOnce>(oop[h], os, 16 * own[h] * pitch, pitch, pitch, lane);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const uint32_t sample = div_by(b, a.H, a.heads_magic);
+    int tv = T;
+    if (t_valid) tv = max(0, min(T, t_valid[sample]));
+    const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
+    RowLane<C> row_lane;
+    TrLane<C> tr_lane;
+    row_lane.init(0, lane);
+    tr_lane.init(0, lane);
+    wait_direct();
+    barrier_lds();
+
+    // ---- queries: delta and dQ -------------------------------------------------------------------------------
+    {
+        RowOperand<C> qop[QT], gop[QT];
+        float dl[QT], lse2[QT];
+        uint32_t drop_key[QT];
+        f32x4 acc[QT][CT];
+#pragma unroll
+        for (int h = 0; h < QT; ++h) {
+            const int qrow = 16 * own[h] + n;
+            read_rows<C>(qop[h], q_lds + own[h] * LL::kTileBytes, row_lane);
+            read_rows<C>(gop[h], g_lds + own[h] * LL::kTileBytes, row_lane);
+            dl[h] = xor_sum(dot_lane<DT, C>(gop[h], oop[h]));       // lane (n, g) holds a quarter of row n's channels
+            lse2[h] = lse_lds[qrow] * kLog2e;
+            if (g == 0) del_lds[qrow] = dl[h];
+            // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dP = D * (dO . V^T) and delta = rowsum(dO * O) as before.
+            drop_key[h] = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) acc[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int kt = 0; kt < TILES; ++kt) {
+            if (kt >= tiles) continue;
+            RowOperand<C> kop, vop;
+            read_rows<C>(kop, k_lds + kt * LL::kTileBytes, row_lane);
+            read_rows<C>(vop, v_lds + kt * LL::kTileBytes, row_lane);
+            u32x2 db[QT];
+#pragma unroll
+            for (int h = 0; h < QT; ++h) {
+                const bool row_masked = 16 * own[h] + n >= tv;
+                const f32x4 sc = dot_rows_mma<DT, C>(kop, qop[h]);
+                const f32x4 dp = dot_rows_mma<DT, C>(vop, gop[h]);
+                float dsv[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int key = 16 * kt + 4 * g + r;
+                    const float z = sc[r] * scale2 - lse2[h] + ((key >= tv || row_masked) ? mask2 : 0.f);
+                    const float p = key < T ? __builtin_amdgcn_exp2f(z) : 0.f;
+                    float dpr = dp[r];
+                    if constexpr (DROP) dpr *= dropout_keeps(drop_key[h], key, a.drop) ? a.drop.inv_keep : 0.f;
+                    dsv[r] = p * (dpr - dl[h]);
+                }
+                db[h] = u32x2{Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
+            }
+            LDS_PTR(char) blk = k_lds + kt * LL::kTileBytes;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const auto kt_t = read_tr(blk + tr_lane.off[ct]);
+#pragma unroll
+                for (int h = 0; h < QT; ++h) acc[h][ct] = Mma<DT>::k16(kt_t, db[h], acc[h][ct]);
+            }
+        }
+        const Rsrc dqs = make_rsrc(dq + seq_off, T * pitch);
+#pragma unroll
+        for (int h = 0; h < QT; ++h) {
+            if (wave + kW * h >= tiles) break;
+            u32x2 qw[CT];
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[h][ct], a.scale);
+            store_tile<C>(dqs, (16 * own[h] + n) * pitch, qw, g, stores_whole_lines(pitch, C, 0), pitch);   // rows past T are dropped
+        }
+    }
+    barrier_lds();                                          // every row's delta is in LDS
+
+    // ---- keys: dK and dV -------------------------------------------------------------------------------------
+    RowOperand<C> kop[QT], vop[QT];
+    f32x4 acck[QT][CT], accv[QT][CT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        read_rows<C>(kop[h], k_lds + own[h] * LL::kTileBytes, row_lane);
+        read_rows<C>(vop[h], v_lds + own[h] * LL::kTileBytes, row_lane);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) acck[h][ct] = accv[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+#pragma unroll
+    for (int qi = 0; qi < TILES; ++qi) {
+        if (qi >= tiles) continue;
+        RowOperand<C> qop, gop;
+        read_rows<C>(qop, q_lds + qi * LL::kTileBytes, row_lane);
+        read_rows<C>(gop, g_lds + qi * LL::kTileBytes, row_lane);
+        const f32x4 lse4 = *reinterpret_cast<LDS_PTR(f32x4)>(lse_lds + 16 * qi + 4 * g);
+        const f32x4 del4 = *reinterpret_cast<LDS_PTR(f32x4)>(del_lds + 16 * qi + 4 * g);
+        u32x2 pb[QT], db[QT];
+#pragma unroll
+        for (int h = 0; h < QT; ++h) {
+            const int key = 16 * own[h] + n;
+            const bool col_masked = key >= tv;
+            const f32x4 sc = dot_rows_mma<DT, C>(qop, kop[h]);       // [query 4g+r][key n]
+            const f32x4 dp = dot_rows_mma<DT, C>(gop, vop[h]);
+            float p[4], dsv[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int qrow = 16 * qi + 4 * g + r;
+                const float z = sc[r] * scale2 - lse4[r] * kLog2e + ((col_masked || qrow >= tv) ? mask2 : 0.f);
+                p[r] = qrow < T ? __builtin_amdgcn_exp2f(z) : 0.f;   // rows past the sequence do not exist
+                float f = 1.f;             // dropout: dP is masked, and dV takes the probability as the forward used it
+                if constexpr (DROP)
+                    f = dropout_keeps(dropout_row_key((uint64_t)b * T + qrow, a.drop), key, a.drop) ? a.drop.inv_keep : 0.f;
+                dsv[r] = p[r] * (dp[r] * f - del4[r]);
+                p[r] *= f;
+            }
+            pb[h] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+            db[h] = u32x2{Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
+        }
+        LDS_PTR(char) qtile = q_lds + qi * LL::kTileBytes;
+        LDS_PTR(char) gtile = g_lds + qi * LL::kTileBytes;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            const auto g_t = read_tr(gtile + tr_lane.off[ct]), q_t = read_tr(qtile + tr_lane.off[ct]);
+#pragma unroll
+            for (int h = 0; h < QT; ++h) {
+                accv[h][ct] = Mma<DT>::k16(g_t, pb[h], accv[h][ct]);
+                acck[h][ct] = Mma<DT>::k16(q_t, db[h], acck[h][ct]);
+            }
+        }
+    }
+    const Rsrc dks = make_rsrc(dk + seq_off, T * pitch), dvs = make_rsrc(dv + seq_off, T * pitch);
+    const bool stream = stores_whole_lines(pitch, C, 0);
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        if (wave + kW * h >= tiles) break;
+        u32x2 kw[CT], vw[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            kw[ct] = pack_acc<DT>(acck[h][ct], a.scale);
+            vw[ct] = pack_acc<DT>(accv[h][ct], 1.f);
+        }
+        store_tile<C>(dks, (16 * own[h] + n) * pitch, kw, g, stream, pitch);      // rows past T are dropped
+        store_tile<C>(dvs, (16 * own[h] + n) * pitch, vw, g, stream, pitch);
+    }
+}
+
 // ----------------------------------------------------------------------------- launchers
 template <int C> constexpr size_t global_lds(int regions) {
     return (size_t)regions * region_bytes<C>(kStripTiles) + 2 * 16 * kStripTiles * sizeof(float);
@@ -418,10 +737,31 @@ int launch_global_fwd(void *out, float *lse, const void *q, const void *k, const
     int64_t items;
     if (!global_ok(g, a, items)) return NA1D_ERR_UNSUPPORTED;
     a.scale = scale;
+    const char *dt_name = DT::tag == NA1D_BF16 ? "BF16" : "FP16", *drop_name = g.drop.threshold ? "true" : "false";
+    if (g.T <= 16 * kShortTiles) {
+        // sequences of up to 4 tiles: 4 waves, a tile each; longer ones: 8 waves, or - with enough sequences to fill
+        // the card several times over - 4 waves of two tiles each, which read every key and value operand half as often
+        const int form = g.T <= 64 ? 0 : g.B < 3 * 256 ? 1 : 2;          // 256 CUs
+        const size_t lds = 2 * (size_t)region_bytes<C>((int)(g.T + 15) / 16);
+        auto go = [&](auto kern, unsigned threads, const char *shape) {
+            if (!allow_lds(kern, lds)) return (int)NA1D_ERR_LAUNCH;
+            note_kernel_as("global_fwd_short_kernel<%s, %d, %s, %s>", dt_name, C, drop_name, shape);
+            launch_kernel_block(kern, (unsigned)g.B, threads, lds, s, (char *)out, lse, (const char *)q, (const char *)k,
+                                (const char *)v, t_valid, a);
+            return launch_status();
+        };
+        if (g.drop.threshold)
+            return form == 0 ? go(global_fwd_short_kernel<DT, C, true, 4, 1>, 256, "4, 1")
+                 : form == 1 ? go(global_fwd_short_kernel<DT, C, true, 8, 1>, 512, "8, 1")
+                             : go(global_fwd_short_kernel<DT, C, true, 8, 2>, 256, "8, 2");
+        return form == 0 ? go(global_fwd_short_kernel<DT, C, false, 4, 1>, 256, "4, 1")
+             : form == 1 ? go(global_fwd_short_kernel<DT, C, false, 8, 1>, 512, "8, 1")
+                         : go(global_fwd_short_kernel<DT, C, false, 8, 2>, 256, "8, 2");
+    }
     auto kern = g.drop.threshold ? global_fwd_kernel<DT, C, true> : global_fwd_kernel<DT, C, false>;
-    if (!allow_lds(kern, global_lds<C>(3))) return NA1D_ERR_LAUNCH;
-    note_kernel_as("global_fwd_kernel<%s, %d, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C, g.drop.threshold ? "true" : "false");
-    launch_kernel(kern, (unsigned)items, global_lds<C>(3), s, (char *)out, lse, (const char *)q, (const char *)k,
+    if (!allow_lds(kern, global_lds<C>(2))) return NA1D_ERR_LAUNCH;
+    note_kernel_as("global_fwd_kernel<%s, %d, %s>", dt_name, C, drop_name);
+    launch_kernel(kern, (unsigned)items, global_lds<C>(2), s, (char *)out, lse, (const char *)q, (const char *)k,
                   (const char *)v, t_valid, (uint32_t)items, a);
     return launch_status();
 }
@@ -434,6 +774,21 @@ int launch_global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q,
     int64_t items;
     if (!global_ok(g, a, items)) return NA1D_ERR_UNSUPPORTED;
     a.scale = scale;
+    if (g.T <= 16 * kShortTiles) {
+        const int tiles_max = g.T <= 64 ? 4 : 8;            // a wave per tile either way
+        const size_t lds = 4 * (size_t)region_bytes<C>((int)(g.T + 15) / 16) + 2 * 16 * tiles_max * sizeof(float);
+        auto go = [&](auto kern) {
+            if (!allow_lds(kern, lds)) return (int)NA1D_ERR_LAUNCH;
+            note_kernel_as("global_bwd_short_kernel<%s, %d, %s, %d, 1>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C,
+                           g.drop.threshold ? "true" : "false", tiles_max);
+            launch_kernel_block(kern, (unsigned)g.B, 64u * tiles_max, lds, s, (char *)dq, (char *)dk, (char *)dv, (const char *)q,
+                                (const char *)k, (const char *)v, (const char *)out, (const char *)dout, lse, t_valid, a);
+            return launch_status();
+        };
+        if (g.drop.threshold)
+            return tiles_max == 4 ? go(global_bwd_short_kernel<DT, C, true, 4, 1>) : go(global_bwd_short_kernel<DT, C, true, 8, 1>);
+        return tiles_max == 4 ? go(global_bwd_short_kernel<DT, C, false, 4, 1>) : go(global_bwd_short_kernel<DT, C, false, 8, 1>);
+    }
     auto dq_kern = g.drop.threshold ? global_dq_kernel<DT, C, true> : global_dq_kernel<DT, C, false>;
     auto dkv_kern = g.drop.threshold ? global_dkv_kernel<DT, C, true> : global_dkv_kernel<DT, C, false>;
     if (!allow_lds(dq_kern, global_lds<C>(5)) || !allow_lds(dkv_kern, global_lds<C>(4))) return NA1D_ERR_LAUNCH;

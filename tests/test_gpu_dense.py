@@ -14,6 +14,10 @@ DTYPES = [torch.bfloat16, torch.float16]
 GEOMS = [  # (N, H, T, C): one tile, ragged tiles, several strips and chunks, every kernel width, padded widths
     (1, 1, 1, 16), (2, 2, 16, 16), (3, 2, 37, 32), (2, 4, 64, 16), (3, 1, 65, 64), (2, 2, 130, 32), (1, 2, 300, 16),
     (2, 1, 129, 128), (2, 2, 100, 24), (1, 3, 77, 48), (2, 1, 90, 104), (1, 1, 1000, 32),
+    # sequences of up to 128 rows take the whole-sequence kernels: at most 4 tiles, 5 to 8 tiles, 8 tiles exactly, and
+    # 768 sequences or more (two query tiles to a wave in the forward)
+    (2, 3, 49, 64), (2, 2, 128, 64), (1, 2, 113, 64), (1, 2, 128, 128), (1, 1, 17, 128), (3, 256, 100, 16),
+    (2, 400, 128, 32), (3, 256, 81, 64),
 ]
 
 
@@ -86,7 +90,8 @@ def test_global_attention_rejects_wide_heads():
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
-@pytest.mark.parametrize("geom", [(2, 2, 37, 32), (1, 3, 130, 64), (2, 1, 100, 24), (1, 2, 300, 16)],
+@pytest.mark.parametrize("geom", [(2, 2, 37, 32), (1, 3, 130, 64), (2, 1, 100, 24), (1, 2, 300, 16), (2, 384, 100, 16),
+                                  (2, 2, 128, 64)],
                          ids=lambda g: "x".join(map(str, g)))
 def test_global_attention_dropout_matches_oracle_with_the_same_mask(geom, dtype):
     N, H, T, C = geom
