@@ -11,6 +11,8 @@
 // a second per key strip computes dK and dV, walking the queries with Q and K swapped in the
 // score product so that the probabilities come out as "lane = key, registers = queries", which
 // is the B operand of dV^T += dO^T P and dK^T += Q^T dS.  No atomics, every output written once.
+#include <type_traits>
+
 #include "na1d_mfma_core.h"
 
 namespace na1d {
@@ -58,7 +60,17 @@ struct GlobalArgs {
 // =============================================================================
 // Forward
 // =============================================================================
-template <class DT, int C, bool DROP>
+// A workgroup owns 4 * QT query tiles, QT to a wave (tiles wave, wave + 4, ...), and walks the keys in chunks of 4
+// tiles that all waves share through LDS; the next chunk is on its way while this one is worked on, so one barrier a
+// chunk.  The wave's query tiles go from memory straight into the registers of the matrix operand.
+//
+// The softmax costs more vector instructions than the two products cost matrix instructions, so a chunk whose keys
+// all count takes a short form: the running maximum comes from the raw products (the scale is made non-negative
+// first, by flipping the sign of the query operand if need be) and scale and maximum fold into one multiply-add in
+// front of the exponential.  Chunks that reach past the valid keys take the long form with its masks.  A padded
+// query row has -100 added to every score: a constant that leaves its probabilities alone and moves its LSE, which
+// is where it is added.
+template <class DT, int C, bool DROP, int QT>
 __global__ void __launch_bounds__(kThreads)
 global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__restrict__ q,
                   const char *__restrict__ k, const char *__restrict__ v, const int32_t *__restrict__ t_valid,
@@ -68,9 +80,8 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     fetch_args_now(out, lse, q, k, v, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic, a.pitch, a.scale);
     if constexpr (DROP) fetch_args_now(a.drop.threshold, a.drop.seed_lo, a.drop.seed_hi, a.drop.inv_keep);
     constexpr int kStep = region_bytes<C>(kStripTiles);
-    extern __shared__ __attribute__((aligned(16))) char smem[];          // 2 * kStep bytes
-    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) v_lds = k_lds + kStep;
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 4 * kStep bytes: K and V of two chunks
+    LDS_PTR(char) kv_lds = (LDS_PTR(char))smem;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -80,96 +91,148 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     const int strip = (int)(item - b * a.strips);
     const uint32_t sample = div_by(b, a.H, a.heads_magic);
     const int T = a.T, tiles = (T + 15) >> 4;
-    const int qt = kStripTiles * strip + wave;              // this wave's query tile
-    const int qrow = 16 * qt + n;
 
     const int64_t seq_off = (int64_t)b * T * a.pitch;
     const Rsrc qs = make_rsrc(q + seq_off, T * a.pitch), ks = make_rsrc(k + seq_off, T * a.pitch);
     const Rsrc vs = make_rsrc(v + seq_off, T * a.pitch), os = make_rsrc(out + seq_off, T * a.pitch);
     const Rsrc ls = make_rsrc(lse ? lse + (int64_t)b * T : nullptr, lse ? T * 4 : 0);
     const int lane_off = direct_lane_offset<C>(wave, lane, a.pitch, a.pitch);
+    stage_direct<C, kStripTiles, kReadShared>(ks, 0, kv_lds, kStripTiles, wave, lane_off, a.pitch);
+    stage_direct<C, kStripTiles, kReadShared>(vs, 0, kv_lds + kStep, kStripTiles, wave, lane_off, a.pitch);
+    int qt[QT];                                             // this wave's query tiles
+    RowOperand<C> qop[QT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        qt[h] = kStripTiles * (QT * strip + h) + wave;
+        load_rows<C, kReadShared>(qop[h], qs, 16 * qt[h] * a.pitch, a.pitch, a.pitch, lane);
+    }
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
-    const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
-    const bool row_masked = qrow >= tv;
+    float scale2 = a.scale * kLog2e;
+    const float mask2 = kMaskValue * kLog2e;
+    if (scale2 < 0.f) {                                     // s * scale = (-s) * (-scale), exactly
+        scale2 = -scale2;
+#pragma unroll
+        for (int h = 0; h < QT; ++h) {
+#pragma unroll
+            for (int s = 0; s < RowOperand<C>::k32; ++s) qop[h].w32[s] ^= 0x80008000u;
+            if (RowOperand<C>::k16) qop[h].w16[0] ^= 0x80008000u;
+        }
+    }
 
     RowLane<C> row_lane;
     TrLane<C> tr_lane;
     row_lane.init(0, lane);
     tr_lane.init(0, lane);
-
-    // the wave's query tile, which no other wave needs, straight into the registers of the matrix operand: a third less
-    // LDS, eight instead of six workgroups on a CU at 64 channels
-    RowOperand<C> qop;
-    load_rows<C, kReadShared>(qop, qs, 16 * qt * a.pitch, a.pitch, a.pitch, lane);
-    float m = kNegInf, l = 0.f;
-    f32x4 o[CT];
+    float m[QT], l[QT];
+    f32x4 o[QT][CT];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) o[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < QT; ++h) {
+        m[h] = kNegInf;
+        l[h] = 0.f;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) o[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 
-    for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
-        if (c0) barrier_lds();                              // every wave is done with the previous chunk
-        stage_direct<C, kStripTiles, kReadShared>(ks, 16 * c0, k_lds, kStripTiles, wave, lane_off, a.pitch);
-        stage_direct<C, kStripTiles, kReadShared>(vs, 16 * c0, v_lds, kStripTiles, wave, lane_off, a.pitch);
-        wait_direct();
-        barrier_lds();
-        const int nk = min(kStripTiles, tiles - c0);        // key tiles in this chunk
-        float z[kStripTiles][4];
-        float mc = kNegInf;
+    // one chunk of keys; `whole`: all of its 64 keys exist and count
+    auto chunk = [&](auto whole, int c0, LDS_PTR(char) k_lds, LDS_PTR(char) v_lds) {
+        constexpr bool kWhole = decltype(whole)::value;
+        const int nk = kWhole ? kStripTiles : min(kStripTiles, tiles - c0);      // key tiles in this chunk
+        f32x4 s[QT][kStripTiles];
 #pragma unroll
         for (int kt = 0; kt < kStripTiles; ++kt) {
             if (kt < nk) {
                 RowOperand<C> kop;
                 read_rows<C>(kop, k_lds + kt * LL::kTileBytes, row_lane);
-                const f32x4 s = dot_rows_mma<DT, C>(kop, qop);
+#pragma unroll
+                for (int h = 0; h < QT; ++h) s[h][kt] = dot_rows_mma<DT, C>(kop, qop[h]);
+            }
+        }
+        u32x2 pb[QT][kStripTiles];
+#pragma unroll
+        for (int h = 0; h < QT; ++h) {
+            const int qrow = 16 * qt[h] + n;
+            const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
+            float mc = kNegInf, m_new;
+            if constexpr (kWhole) {
+#pragma unroll
+                for (int kt = 0; kt < kStripTiles; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) mc = __builtin_fmaxf(mc, s[h][kt][r]);
+                m_new = max2(m[h], xor_max(mc) * scale2);
+            } else {
+                const bool row_masked = qrow >= tv;
+#pragma unroll
+                for (int kt = 0; kt < kStripTiles; ++kt)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = 16 * (c0 + kt) + 4 * g + r;
+                        const float zz = s[h][kt][r] * scale2 + ((key >= tv && !row_masked) ? mask2 : 0.f);
+                        s[h][kt][r] = kt < nk && key < T ? zz : kNegInf;      // rows past the sequence do not exist
+                        mc = __builtin_fmaxf(mc, s[h][kt][r]);
+                    }
+                m_new = max2(m[h], xor_max(mc));            // finite: key 16 * c0 exists
+            }
+            const float alpha = __builtin_amdgcn_exp2f(m[h] - m_new);
+            float part = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < kStripTiles; ++kt) {
+                float p[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    const int key = 16 * (c0 + kt) + 4 * g + r;
-                    float zz = s[r] * scale2 + ((key >= tv || row_masked) ? mask2 : 0.f);
-                    z[kt][r] = key < T ? zz : kNegInf;      // rows past the sequence do not exist
+                    p[r] = __builtin_amdgcn_exp2f(kWhole ? __builtin_fmaf(s[h][kt][r], scale2, -m_new) : s[h][kt][r] - m_new);
+                    part += p[r];
+                    // a dropped probability stays in the sum and leaves O
+                    if (DROP && !dropout_keeps(drop_key, 16 * (c0 + kt) + 4 * g + r, a.drop)) p[r] = 0.f;
                 }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 4; ++r) z[kt][r] = kNegInf;
+                pb[h][kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
             }
-            mc = max3(mc, max2(z[kt][0], z[kt][1]), max2(z[kt][2], z[kt][3]));
+            l[h] = l[h] * alpha + xor_sum(part);
+            m[h] = m_new;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) o[h][ct] = o[h][ct] * alpha;
         }
-        const float m_new = max2(m, xor_max(mc));           // finite: key 16*c0 exists
-        const float alpha = __builtin_amdgcn_exp2f(m - m_new);
-        float part = 0.f;
-        u32x2 pb[kStripTiles];
-        const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
-#pragma unroll
-        for (int kt = 0; kt < kStripTiles; ++kt) {
-            float p[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(z[kt][r] - m_new);
-                part += p[r];
-                // a dropped probability stays in the sum and leaves O
-                if (DROP && !dropout_keeps(drop_key, 16 * (c0 + kt) + 4 * g + r, a.drop)) p[r] = 0.f;
-            }
-            pb[kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
-        }
-        l = l * alpha + xor_sum(part);
-        m = m_new;
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) o[ct] = o[ct] * alpha;
 #pragma unroll
         for (int kt = 0; kt < kStripTiles; ++kt) {
             if (kt >= nk) continue;
             LDS_PTR(char) blk = v_lds + kt * LL::kTileBytes;
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) o[ct] = Mma<DT>::k16(read_tr(blk + tr_lane.off[ct]), pb[kt], o[ct]);
-        }
-    }
-    if (qt >= tiles) return;                                // after the last barrier
-    const float inv = __builtin_amdgcn_rcpf(l) * (DROP ? a.drop.inv_keep : 1.f);
-    u32x2 ow[CT];
+            for (int ct = 0; ct < CT; ++ct) {
+                const u32x2 vt = read_tr(blk + tr_lane.off[ct]);
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[ct], inv);
-    store_tile<C>(os, qrow * a.pitch, ow, g, stores_whole_lines(a.pitch, C, 0), a.pitch);   // rows past T are dropped
-    if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint((m + __builtin_amdgcn_logf(l)) * kLn2), ls, qrow * 4, 0, 0);
+                for (int h = 0; h < QT; ++h) o[h][ct] = Mma<DT>::k16(vt, pb[h][kt], o[h][ct]);
+            }
+        }
+    };
+
+    const int whole_keys = min(T, tv);
+    int at = 0;                                             // byte offset of the chunk's pair of regions: 0 or 2 * kStep
+    for (int c0 = 0; c0 < tiles; c0 += kStripTiles, at ^= 2 * kStep) {
+        wait_direct();
+        barrier_lds();      // this chunk has landed, and every wave is done with the one before, whose regions the next takes
+        if (c0 + kStripTiles < tiles) {
+            LDS_PTR(char) next = kv_lds + (at ^ 2 * kStep);
+            stage_direct<C, kStripTiles, kReadShared>(ks, 16 * (c0 + kStripTiles), next, kStripTiles, wave, lane_off, a.pitch);
+            stage_direct<C, kStripTiles, kReadShared>(vs, 16 * (c0 + kStripTiles), next + kStep, kStripTiles, wave, lane_off, a.pitch);
+        }
+        if (16 * (c0 + kStripTiles) <= whole_keys)
+            chunk(std::true_type{}, c0, kv_lds + at, kv_lds + at + kStep);
+        else
+            chunk(std::false_type{}, c0, kv_lds + at, kv_lds + at + kStep);
+    }
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        if (qt[h] >= tiles) break;
+        const int qrow = 16 * qt[h] + n;
+        const float inv = __builtin_amdgcn_rcpf(l[h]) * (DROP ? a.drop.inv_keep : 1.f);
+        u32x2 ow[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[h][ct], inv);
+        store_tile<C>(os, qrow * a.pitch, ow, g, stores_whole_lines(a.pitch, C, 0), a.pitch);   // rows past T are dropped
+        const float pad = qrow >= tv ? kMaskValue : 0.f;
+        if (g == 0)
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint((m[h] + __builtin_amdgcn_logf(l[h])) * kLn2 + pad), ls, qrow * 4, 0, 0);
+    }
 }
 
 // =============================================================================
@@ -758,12 +821,24 @@ int launch_global_fwd(void *out, float *lse, const void *q, const void *k, const
              : form == 1 ? go(global_fwd_short_kernel<DT, C, false, 8, 1>, 512, "8, 1")
                          : go(global_fwd_short_kernel<DT, C, false, 8, 2>, 256, "8, 2");
     }
-    auto kern = g.drop.threshold ? global_fwd_kernel<DT, C, true> : global_fwd_kernel<DT, C, false>;
-    if (!allow_lds(kern, global_lds<C>(2))) return NA1D_ERR_LAUNCH;
-    note_kernel_as("global_fwd_kernel<%s, %d, %s>", dt_name, C, drop_name);
-    launch_kernel(kern, (unsigned)items, global_lds<C>(2), s, (char *)out, lse, (const char *)q, (const char *)k,
-                  (const char *)v, t_valid, (uint32_t)items, a);
-    return launch_status();
+    // two query tiles to a wave where that still leaves every CU several workgroups
+    const int64_t strips2 = (a.strips + 1) / 2;
+    const bool two = g.B * strips2 >= 4 * 256 && div_magic_ok(g.B * strips2, strips2);
+    if (two) {
+        a.strips = (int)strips2;
+        a.strips_magic = div_magic(a.strips);
+        items = g.B * strips2;
+    }
+    const size_t lds = 4 * (size_t)region_bytes<C>(kStripTiles);
+    auto go = [&](auto kern) {
+        if (!allow_lds(kern, lds)) return (int)NA1D_ERR_LAUNCH;
+        note_kernel_as("global_fwd_kernel<%s, %d, %s, %d>", dt_name, C, drop_name, two ? 2 : 1);
+        launch_kernel(kern, (unsigned)items, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v, t_valid,
+                      (uint32_t)items, a);
+        return launch_status();
+    };
+    if (g.drop.threshold) return two ? go(global_fwd_kernel<DT, C, true, 2>) : go(global_fwd_kernel<DT, C, true, 1>);
+    return two ? go(global_fwd_kernel<DT, C, false, 2>) : go(global_fwd_kernel<DT, C, false, 1>);
 }
 
 template <class DT, int C>
