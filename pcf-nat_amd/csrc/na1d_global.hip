@@ -124,12 +124,14 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     TrLane<C> tr_lane;
     row_lane.init(0, lane);
     tr_lane.init(0, lane);
+    constexpr float kSlack = 6.f;
     float m[QT], l[QT];
-    f32x4 o[QT][CT];
+    f32x4 o[QT][CT], lsum[QT];                              // lsum: the row sum in every register, without dropout
 #pragma unroll
     for (int h = 0; h < QT; ++h) {
         m[h] = kNegInf;
         l[h] = 0.f;
+        lsum[h] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) o[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
@@ -148,18 +150,18 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
                 for (int h = 0; h < QT; ++h) s[h][kt] = dot_rows_mma<DT, C>(kop, qop[h]);
             }
         }
-        u32x2 pb[QT][kStripTiles];
+        u32x4 pp[QT][kStripTiles / 2];          // probabilities of two key tiles: the B operand of a 32-deep product
 #pragma unroll
         for (int h = 0; h < QT; ++h) {
             const int qrow = 16 * qt[h] + n;
             const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
-            float mc = kNegInf, m_new;
+            float mc = kNegInf;
             if constexpr (kWhole) {
 #pragma unroll
                 for (int kt = 0; kt < kStripTiles; ++kt)
 #pragma unroll
                     for (int r = 0; r < 4; ++r) mc = __builtin_fmaxf(mc, s[h][kt][r]);
-                m_new = max2(m[h], xor_max(mc) * scale2);
+                mc = xor_max(mc) * scale2;
             } else {
                 const bool row_masked = qrow >= tv;
 #pragma unroll
@@ -171,36 +173,57 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
                         s[h][kt][r] = kt < nk && key < T ? zz : kNegInf;      // rows past the sequence do not exist
                         mc = __builtin_fmaxf(mc, s[h][kt][r]);
                     }
-                m_new = max2(m[h], xor_max(mc));            // finite: key 16 * c0 exists
+                mc = xor_max(mc);                           // finite: key 16 * c0 exists
             }
-            const float alpha = __builtin_amdgcn_exp2f(m[h] - m_new);
+            // The reference point of the exponentials moves only when a row's maximum has outgrown it by more than
+            // kSlack (probabilities then stay below 2^kSlack, which every format here holds): most chunks leave
+            // the accumulators as they are.
+            if (__builtin_amdgcn_ballot_w64(mc > m[h] + kSlack)) {
+                const float m_new = max2(m[h], mc);
+                const float alpha = __builtin_amdgcn_exp2f(m[h] - m_new);
+                m[h] = m_new;
+                l[h] *= alpha;
+                if constexpr (!DROP) lsum[h] = lsum[h] * alpha;
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) o[h][ct] = o[h][ct] * alpha;
+            }
+            const float ref = -m[h];
             float part = 0.f;
 #pragma unroll
             for (int kt = 0; kt < kStripTiles; ++kt) {
                 float p[4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    p[r] = __builtin_amdgcn_exp2f(kWhole ? __builtin_fmaf(s[h][kt][r], scale2, -m_new) : s[h][kt][r] - m_new);
-                    part += p[r];
-                    // a dropped probability stays in the sum and leaves O
-                    if (DROP && !dropout_keeps(drop_key, 16 * (c0 + kt) + 4 * g + r, a.drop)) p[r] = 0.f;
+                    p[r] = __builtin_amdgcn_exp2f(kWhole ? __builtin_fmaf(s[h][kt][r], scale2, ref) : s[h][kt][r] + ref);
+                    if constexpr (DROP) {                   // a dropped probability stays in the sum and leaves O
+                        part += p[r];
+                        if (!dropout_keeps(drop_key, 16 * (c0 + kt) + 4 * g + r, a.drop)) p[r] = 0.f;
+                    }
                 }
-                pb[h][kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+                pp[h][kt / 2][2 * (kt & 1)] = Mma<DT>::pack(p[0], p[1]);
+                pp[h][kt / 2][2 * (kt & 1) + 1] = Mma<DT>::pack(p[2], p[3]);
             }
-            l[h] = l[h] * alpha + xor_sum(part);
-            m[h] = m_new;
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) o[h][ct] = o[h][ct] * alpha;
+            if constexpr (DROP) l[h] += xor_sum(part);
         }
+        // O^T += V^T P^T over two key tiles at a time (the 32-deep product costs what the 16-deep one does); a tile
+        // past the chunk's last has zero probabilities and zeros in LDS.  Without dropout the row sums come from
+        // the same instruction with ones in place of V^T.
 #pragma unroll
-        for (int kt = 0; kt < kStripTiles; ++kt) {
+        for (int kt = 0; kt < kStripTiles; kt += 2) {
             if (kt >= nk) continue;
             LDS_PTR(char) blk = v_lds + kt * LL::kTileBytes;
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                const u32x2 vt = read_tr(blk + tr_lane.off[ct]);
+                const u32x2 v0 = read_tr(blk + tr_lane.off[ct]), v1 = read_tr(blk + LL::kTileBytes + tr_lane.off[ct]);
+                const u32x4 vv = {v0.x, v0.y, v1.x, v1.y};
 #pragma unroll
-                for (int h = 0; h < QT; ++h) o[h][ct] = Mma<DT>::k16(vt, pb[h][kt], o[h][ct]);
+                for (int h = 0; h < QT; ++h) o[h][ct] = Mma<DT>::k32(vv, pp[h][kt / 2], o[h][ct]);
+            }
+            if constexpr (!DROP) {
+                const uint32_t one = Mma<DT>::pack(1.f, 1.f);
+                const u32x4 ones = {one, one, one, one};
+#pragma unroll
+                for (int h = 0; h < QT; ++h) lsum[h] = Mma<DT>::k32(ones, pp[h][kt / 2], lsum[h]);
             }
         }
     };
@@ -224,6 +247,7 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     for (int h = 0; h < QT; ++h) {
         if (qt[h] >= tiles) break;
         const int qrow = 16 * qt[h] + n;
+        if constexpr (!DROP) l[h] = lsum[h][0];
         const float inv = __builtin_amdgcn_rcpf(l[h]) * (DROP ? a.drop.inv_keep : 1.f);
         u32x2 ow[CT];
 #pragma unroll
