@@ -49,6 +49,17 @@ __device__ inline float dot_lane(const RowOperand<C> &a, const RowOperand<C> &b)
     return acc;
 }
 
+// x *= a in the registers x lives in.  Written as plain C++ inside a branch, the compiler gives the products new
+// registers and pays for it with copies of every accumulator on both sides of the branch.  The accumulators are
+// results of matrix instructions the compiler cannot relate to this block: callers keep at least a dozen
+// instructions between the last of those and this.  The factor may come straight out of a transcendental
+// instruction, whose result an ordinary vector instruction may read one state later at the earliest: hence the s_nop.
+__device__ inline void scale_in_place(f32x4 &x, float a) {
+    asm volatile("s_nop 0\n\tv_mul_f32 %0, %4, %0\n\tv_mul_f32 %1, %4, %1\n\tv_mul_f32 %2, %4, %2\n\tv_mul_f32 %3, %4, %3"
+                 : "+v"(x[0]), "+v"(x[1]), "+v"(x[2]), "+v"(x[3])
+                 : "v"(a));
+}
+
 struct GlobalArgs {
     int T, H, strips;            // strips of kStripTiles tiles per sequence
     uint32_t strips_magic, heads_magic;
@@ -183,9 +194,9 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
                 const float alpha = __builtin_amdgcn_exp2f(m[h] - m_new);
                 m[h] = m_new;
                 l[h] *= alpha;
-                if constexpr (!DROP) lsum[h] = lsum[h] * alpha;
+                if constexpr (!DROP) scale_in_place(lsum[h], alpha);
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) o[h][ct] = o[h][ct] * alpha;
+                for (int ct = 0; ct < CT; ++ct) scale_in_place(o[h][ct], alpha);
             }
             const float ref = -m[h];
             float part = 0.f;
@@ -228,9 +239,11 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
         }
     };
 
+    // Chunks whose keys all count come first and have a loop of their own: with both forms in one loop body the
+    // accumulators change registers where the two meet, at the price of a copy of each per chunk.
     const int whole_keys = min(T, tv);
     int at = 0;                                             // byte offset of the chunk's pair of regions: 0 or 2 * kStep
-    for (int c0 = 0; c0 < tiles; c0 += kStripTiles, at ^= 2 * kStep) {
+    auto step = [&](auto whole, int c0) {
         wait_direct();
         barrier_lds();      // this chunk has landed, and every wave is done with the one before, whose regions the next takes
         if (c0 + kStripTiles < tiles) {
@@ -238,11 +251,12 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
             stage_direct<C, kStripTiles, kReadShared>(ks, 16 * (c0 + kStripTiles), next, kStripTiles, wave, lane_off, a.pitch);
             stage_direct<C, kStripTiles, kReadShared>(vs, 16 * (c0 + kStripTiles), next + kStep, kStripTiles, wave, lane_off, a.pitch);
         }
-        if (16 * (c0 + kStripTiles) <= whole_keys)
-            chunk(std::true_type{}, c0, kv_lds + at, kv_lds + at + kStep);
-        else
-            chunk(std::false_type{}, c0, kv_lds + at, kv_lds + at + kStep);
-    }
+        chunk(whole, c0, kv_lds + at, kv_lds + at + kStep);
+        at ^= 2 * kStep;
+    };
+    int c0 = 0;
+    for (; 16 * (c0 + kStripTiles) <= whole_keys; c0 += kStripTiles) step(std::true_type{}, c0);
+    for (; c0 < tiles; c0 += kStripTiles) step(std::false_type{}, c0);
 #pragma unroll
     for (int h = 0; h < QT; ++h) {
         if (qt[h] >= tiles) break;
