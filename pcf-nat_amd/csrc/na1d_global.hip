@@ -321,21 +321,33 @@ global_fwd_short_kernel(char *__restrict__ out, float *__restrict__ lse, const c
     wait_direct();
     barrier_lds();
 
+    // Scores of all keys, in the log2 domain.  A tile whose 16 keys all count needs the scale only; a padded query
+    // row has -100 added to every score, which leaves its probabilities alone and moves its LSE: added there.
+    const int whole_keys = min(T, tv);
     float z[QT][TILES][4];
 #pragma unroll
     for (int kt = 0; kt < TILES; ++kt) {
         if (kt < tiles) {
             RowOperand<C> kop;
             read_rows<C>(kop, k_lds + kt * LL::kTileBytes, row_lane);
+            f32x4 s[QT];
 #pragma unroll
-            for (int h = 0; h < QT; ++h) {
-                const bool row_masked = 16 * (wave + kW * h) + n >= tv;
-                const f32x4 s = dot_rows_mma<DT, C>(kop, qop[h]);
+            for (int h = 0; h < QT; ++h) s[h] = dot_rows_mma<DT, C>(kop, qop[h]);
+            if (16 * (kt + 1) <= whole_keys) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int key = 16 * kt + 4 * g + r;
-                    const float zz = s[r] * scale2 + ((key >= tv || row_masked) ? mask2 : 0.f);
-                    z[h][kt][r] = key < T ? zz : kNegInf;   // rows past the sequence do not exist
+                for (int h = 0; h < QT; ++h)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) z[h][kt][r] = s[h][r] * scale2;
+            } else {
+#pragma unroll
+                for (int h = 0; h < QT; ++h) {
+                    const bool row_masked = 16 * (wave + kW * h) + n >= tv;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int key = 16 * kt + 4 * g + r;
+                        const float zz = s[h][r] * scale2 + ((key >= tv && !row_masked) ? mask2 : 0.f);
+                        z[h][kt][r] = key < T ? zz : kNegInf;   // rows past the sequence do not exist
+                    }
                 }
             }
         } else {
@@ -344,6 +356,8 @@ global_fwd_short_kernel(char *__restrict__ out, float *__restrict__ lse, const c
 #pragma unroll
                 for (int r = 0; r < 4; ++r) z[h][kt][r] = kNegInf;
         }
+        // left alone, the scheduler reads every key tile before the first product and runs out of registers
+        if (kt & 1) __builtin_amdgcn_sched_barrier(0);
     }
     u32x2 pb[QT][TILES];
     float m[QT], l[QT];
@@ -358,44 +372,77 @@ global_fwd_short_kernel(char *__restrict__ out, float *__restrict__ lse, const c
         float part = 0.f;
 #pragma unroll
         for (int kt = 0; kt < TILES; ++kt) {
-            float p[4];
+            if (kt < tiles) {
+                float p[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(z[h][kt][r] - m[h]);
-                part += p[r];
-                // a dropped probability stays in the sum and leaves O
-                if (DROP && !dropout_keeps(drop_key, 16 * kt + 4 * g + r, a.drop)) p[r] = 0.f;
+                for (int r = 0; r < 4; ++r) {
+                    p[r] = __builtin_amdgcn_exp2f(z[h][kt][r] - m[h]);
+                    if constexpr (DROP) {                   // a dropped probability stays in the sum and leaves O
+                        part += p[r];
+                        if (!dropout_keeps(drop_key, 16 * kt + 4 * g + r, a.drop)) p[r] = 0.f;
+                    }
+                }
+                pb[h][kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
+            } else {
+                pb[h][kt] = u32x2{0u, 0u};
             }
-            pb[h][kt] = u32x2{Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
         }
-        l[h] = xor_sum(part);
+        l[h] = DROP ? xor_sum(part) : 0.f;
     }
-    f32x4 o[QT][CT];
+    // O^T = V^T P^T, two key tiles to a 32-deep product (a last single tile: 16-deep).  Without dropout the row sums
+    // come from the same instruction with ones in place of V^T.
+    f32x4 o[QT][CT], lsum[QT];
 #pragma unroll
-    for (int h = 0; h < QT; ++h)
+    for (int h = 0; h < QT; ++h) {
+        lsum[h] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) o[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    const uint32_t one = Mma<DT>::pack(1.f, 1.f);
 #pragma unroll
-    for (int kt = 0; kt < TILES; ++kt) {
+    for (int kt = 0; kt < TILES; kt += 2) {
         if (kt >= tiles) continue;
         LDS_PTR(char) blk = v_lds + kt * LL::kTileBytes;
+        if (kt + 1 < tiles) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            const auto vt = read_tr(blk + tr_lane.off[ct]);
+            for (int ct = 0; ct < CT; ++ct) {
+                const u32x2 v0 = read_tr(blk + tr_lane.off[ct]), v1 = read_tr(blk + LL::kTileBytes + tr_lane.off[ct]);
+                const u32x4 vv = {v0.x, v0.y, v1.x, v1.y};
 #pragma unroll
-            for (int h = 0; h < QT; ++h) o[h][ct] = Mma<DT>::k16(vt, pb[h][kt], o[h][ct]);
+                for (int h = 0; h < QT; ++h)
+                    o[h][ct] = Mma<DT>::k32(vv, u32x4{pb[h][kt].x, pb[h][kt].y, pb[h][kt + 1].x, pb[h][kt + 1].y}, o[h][ct]);
+            }
+            if constexpr (!DROP)
+#pragma unroll
+                for (int h = 0; h < QT; ++h)
+                    lsum[h] = Mma<DT>::k32(u32x4{one, one, one, one},
+                                           u32x4{pb[h][kt].x, pb[h][kt].y, pb[h][kt + 1].x, pb[h][kt + 1].y}, lsum[h]);
+        } else {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const u32x2 vt = read_tr(blk + tr_lane.off[ct]);
+#pragma unroll
+                for (int h = 0; h < QT; ++h) o[h][ct] = Mma<DT>::k16(vt, pb[h][kt], o[h][ct]);
+            }
+            if constexpr (!DROP)
+#pragma unroll
+                for (int h = 0; h < QT; ++h) lsum[h] = Mma<DT>::k16(u32x2{one, one}, pb[h][kt], lsum[h]);
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
     for (int h = 0; h < QT; ++h) {
         if (wave + kW * h >= tiles) break;
         const int qrow = 16 * (wave + kW * h) + n;
+        if constexpr (!DROP) l[h] = lsum[h][0];
         const float inv = __builtin_amdgcn_rcpf(l[h]) * (DROP ? a.drop.inv_keep : 1.f);
         u32x2 ow[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) ow[ct] = pack_acc<DT>(o[h][ct], inv);
         store_tile<C>(os, qrow * pitch, ow, g, stores_whole_lines(pitch, C, 0), pitch);     // rows past T are dropped
-        if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint((m[h] + __builtin_amdgcn_logf(l[h])) * kLn2), ls, qrow * 4, 0, 0);
+        const float pad = qrow >= tv ? kMaskValue : 0.f;
+        if (g == 0)
+            __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint((m[h] + __builtin_amdgcn_logf(l[h])) * kLn2 + pad), ls, qrow * 4, 0, 0);
     }
 }
 
@@ -840,24 +887,20 @@ int launch_global_fwd(void *out, float *lse, const void *q, const void *k, const
     a.scale = scale;
     const char *dt_name = DT::tag == NA1D_BF16 ? "BF16" : "FP16", *drop_name = g.drop.threshold ? "true" : "false";
     if (g.T <= 16 * kShortTiles) {
-        // sequences of up to 4 tiles: 4 waves, a tile each; longer ones: 8 waves, or - with enough sequences to fill
-        // the card several times over - 4 waves of two tiles each, which read every key and value operand half as often
-        const int form = g.T <= 64 ? 0 : g.B < 3 * 256 ? 1 : 2;          // 256 CUs
+        // sequences of up to 4 tiles: a tile to each of the 4 waves; longer ones: two, which read every key and value
+        // operand half as often
+        const bool small = g.T <= 64;
         const size_t lds = 2 * (size_t)region_bytes<C>((int)(g.T + 15) / 16);
-        auto go = [&](auto kern, unsigned threads, const char *shape) {
+        auto go = [&](auto kern) {
             if (!allow_lds(kern, lds)) return (int)NA1D_ERR_LAUNCH;
-            note_kernel_as("global_fwd_short_kernel<%s, %d, %s, %s>", dt_name, C, drop_name, shape);
-            launch_kernel_block(kern, (unsigned)g.B, threads, lds, s, (char *)out, lse, (const char *)q, (const char *)k,
-                                (const char *)v, t_valid, a);
+            note_kernel_as("global_fwd_short_kernel<%s, %d, %s, %s>", dt_name, C, drop_name, small ? "4, 1" : "8, 2");
+            launch_kernel(kern, (unsigned)g.B, lds, s, (char *)out, lse, (const char *)q, (const char *)k, (const char *)v,
+                          t_valid, a);
             return launch_status();
         };
         if (g.drop.threshold)
-            return form == 0 ? go(global_fwd_short_kernel<DT, C, true, 4, 1>, 256, "4, 1")
-                 : form == 1 ? go(global_fwd_short_kernel<DT, C, true, 8, 1>, 512, "8, 1")
-                             : go(global_fwd_short_kernel<DT, C, true, 8, 2>, 256, "8, 2");
-        return form == 0 ? go(global_fwd_short_kernel<DT, C, false, 4, 1>, 256, "4, 1")
-             : form == 1 ? go(global_fwd_short_kernel<DT, C, false, 8, 1>, 512, "8, 1")
-                         : go(global_fwd_short_kernel<DT, C, false, 8, 2>, 256, "8, 2");
+            return small ? go(global_fwd_short_kernel<DT, C, true, 4, 1>) : go(global_fwd_short_kernel<DT, C, true, 8, 2>);
+        return small ? go(global_fwd_short_kernel<DT, C, false, 4, 1>) : go(global_fwd_short_kernel<DT, C, false, 8, 2>);
     }
     // two query tiles to a wave where that still leaves every CU several workgroups
     const int64_t strips2 = (a.strips + 1) / 2;

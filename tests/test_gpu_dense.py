@@ -15,7 +15,7 @@ GEOMS = [  # (N, H, T, C): one tile, ragged tiles, several strips and chunks, ev
     (1, 1, 1, 16), (2, 2, 16, 16), (3, 2, 37, 32), (2, 4, 64, 16), (3, 1, 65, 64), (2, 2, 130, 32), (1, 2, 300, 16),
     (2, 1, 129, 128), (2, 2, 100, 24), (1, 3, 77, 48), (2, 1, 90, 104), (1, 1, 1000, 32),
     # sequences of up to 128 rows take the whole-sequence kernels: at most 4 tiles, 5 to 8 tiles, 8 tiles exactly, and
-    # 768 sequences or more (two query tiles to a wave in the forward)
+    # launches of many sequences
     (2, 3, 49, 64), (2, 2, 128, 64), (1, 2, 113, 64), (1, 2, 128, 128), (1, 1, 17, 128), (3, 256, 100, 16),
     (2, 400, 128, 32), (3, 256, 81, 64),
 ]
