@@ -231,7 +231,8 @@ int na1d_fused_backward_strided_dropout(void *dq, void *dk, void *dv, float *drp
  * q, k, v, out and the gradients are packed [B, T, C] with B = samples * H, head fastest inside a sample;
  * lse [B, T] fp32 (natural log; may be NULL in the forward when no backward follows).  The probabilities are never
  * written to memory.  The backward needs a workspace of na1d_global_backward_workspace_bytes() bytes (one fp32 per
- * row: rowsum(dout * out)) and writes every gradient exactly once, so it is deterministic.
+ * row: rowsum(dout * out); sequences of up to 128 rows keep it on chip and leave the workspace untouched) and writes
+ * every gradient exactly once, so it is deterministic.
  * C % 8 == 0; C > 128 returns NA1D_ERR_UNSUPPORTED.  scale: finite and > 0 as in na1d_fused_forward.  p_drop, seed: attention dropout (attn_drop of
  * models/PCF_NATransformer.py:193,218; 0 in the reference's configurations) by the keep rule stated at
  * na1d_fused_forward_dropout with the key's row index as the slot j; 0 <= p_drop < 1, 0 switches it off.

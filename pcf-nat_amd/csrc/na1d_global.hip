@@ -5,9 +5,12 @@
 // softmax whose row statistics are lane-local up to a reduction over the four lane groups, and
 // the rounded probabilities fed straight back as the B operand of O^T += V^T P^T.
 //
-// Forward: a workgroup owns 4 query tiles (one per wave) and walks the keys in chunks of 4 tiles
-// that all four waves share through LDS.
-// Backward: one kernel per query strip computes delta = rowsum(dO * O) and dQ, walking the keys;
+// Sequences of up to 128 rows (the models run at about 100): one workgroup per sequence with everything it needs whole
+// in LDS behind one barrier - a forward with a plain softmax, and a backward that is ONE kernel (delta never leaves the
+// chip, every input is read once).
+// Longer sequences: the forward owns 4 or 8 query tiles per workgroup (one or two per wave) and walks the keys in
+// chunks of 4 tiles that all four waves share through LDS, the next chunk in flight behind the current one.
+// Their backward: one kernel per query strip computes delta = rowsum(dO * O) and dQ, walking the keys;
 // a second per key strip computes dK and dV, walking the queries with Q and K swapped in the
 // score product so that the probabilities come out as "lane = key, registers = queries", which
 // is the B operand of dV^T += dO^T P and dK^T += Q^T dS.  No atomics, every output written once.
@@ -76,9 +79,8 @@ struct GlobalArgs {
 // chunk.  The wave's query tiles go from memory straight into the registers of the matrix operand.
 //
 // The softmax costs more vector instructions than the two products cost matrix instructions, so a chunk whose keys
-// all count takes a short form: the running maximum comes from the raw products (the scale is made non-negative
-// first, by flipping the sign of the query operand if need be) and scale and maximum fold into one multiply-add in
-// front of the exponential.  Chunks that reach past the valid keys take the long form with its masks.  A padded
+// all count takes a short form: the running maximum comes from the raw products (the scale is positive) and scale
+// and maximum fold into one multiply-add in front of the exponential.  Chunks that reach past the valid keys take the long form with its masks.  A padded
 // query row has -100 added to every score: a constant that leaves its probabilities alone and moves its LSE, which
 // is where it is added.
 template <class DT, int C, bool DROP, int QT>
@@ -119,17 +121,7 @@ global_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *_
     }
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
-    float scale2 = a.scale * kLog2e;
-    const float mask2 = kMaskValue * kLog2e;
-    if (scale2 < 0.f) {                                     // s * scale = (-s) * (-scale), exactly
-        scale2 = -scale2;
-#pragma unroll
-        for (int h = 0; h < QT; ++h) {
-#pragma unroll
-            for (int s = 0; s < RowOperand<C>::k32; ++s) qop[h].w32[s] ^= 0x80008000u;
-            if (RowOperand<C>::k16) qop[h].w16[0] ^= 0x80008000u;
-        }
-    }
+    const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;     // the scale is positive: checked at the C boundary
 
     RowLane<C> row_lane;
     TrLane<C> tr_lane;
