@@ -441,7 +441,11 @@ global_fwd_short_kernel(char *__restrict__ out, float *__restrict__ lse, const c
 // =============================================================================
 // Backward, query side: delta = rowsum(dO * O) (written to `delta`) and dQ
 // =============================================================================
-template <class DT, int C, bool DROP>
+// A workgroup owns 4 * QT query tiles, QT to a wave, whose Q, dO and O rows go from memory straight into registers,
+// and walks the keys in chunks of 4 tiles (K and V through LDS, the next chunk in flight behind the current one).
+// dQ^T += K^T dS^T runs two key tiles at a time on the 32-deep product.  A padded query row's -100 is folded into
+// its LSE once; chunks whose keys all count skip the masks.
+template <class DT, int C, bool DROP, int QT>
 __global__ void __launch_bounds__(kThreads)
 global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *__restrict__ q,
                  const char *__restrict__ k, const char *__restrict__ v, const char *__restrict__ out,
@@ -452,12 +456,9 @@ global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *_
     constexpr int kStep = region_bytes<C>(kStripTiles);
     fetch_args_now(dq, delta, q, k, v, out, dout, lse, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic,
                    a.pitch, a.scale);
-    extern __shared__ __attribute__((aligned(16))) char smem[];          // 5 * kStep bytes
-    LDS_PTR(char) q_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) g_lds = q_lds + kStep;                    // dO
-    LDS_PTR(char) o_lds = g_lds + kStep;
-    LDS_PTR(char) k_lds = o_lds + kStep;
-    LDS_PTR(char) v_lds = k_lds + kStep;
+    if constexpr (DROP) fetch_args_now(a.drop.threshold, a.drop.seed_lo, a.drop.seed_hi, a.drop.inv_keep);
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 4 * kStep bytes: K and V of two chunks
+    LDS_PTR(char) kv_lds = (LDS_PTR(char))smem;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -467,8 +468,6 @@ global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *_
     const int strip = (int)(item - b * a.strips);
     const uint32_t sample = div_by(b, a.H, a.heads_magic);
     const int T = a.T, tiles = (T + 15) >> 4;
-    const int qt = kStripTiles * strip + wave;
-    const int qrow = 16 * qt + n;
 
     const int64_t seq_off = (int64_t)b * T * a.pitch;
     const Rsrc qs = make_rsrc(q + seq_off, T * a.pitch), ks = make_rsrc(k + seq_off, T * a.pitch);
@@ -476,79 +475,129 @@ global_dq_kernel(char *__restrict__ dq, float *__restrict__ delta, const char *_
     const Rsrc gs = make_rsrc(dout + seq_off, T * a.pitch), dqs = make_rsrc(dq + seq_off, T * a.pitch);
     const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4), ds = make_rsrc(delta + (int64_t)b * T, T * 4);
     const int lane_off = direct_lane_offset<C>(wave, lane, a.pitch, a.pitch);
+    stage_direct<C, kStripTiles, kReadShared>(ks, 0, kv_lds, kStripTiles, wave, lane_off, a.pitch);
+    stage_direct<C, kStripTiles, kReadShared>(vs, 0, kv_lds + kStep, kStripTiles, wave, lane_off, a.pitch);
+    int qt[QT];                                             // this wave's query tiles
+    RowOperand<C> qop[QT], gop[QT], oop[QT];
+    float lse_row[QT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        qt[h] = kStripTiles * (QT * strip + h) + wave;
+        const int at = 16 * qt[h] * a.pitch;
+        load_rows<C, kReadShared>(qop[h], qs, at, a.pitch, a.pitch, lane);
+        load_rows<C, kReadShared>(gop[h], gs, at, a.pitch, a.pitch, lane);
+        load_rows<C, kReadOnce>(oop[h], os, at, a.pitch, a.pitch, lane);
+        lse_row[h] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ls, (16 * qt[h] + n) * 4, 0, 0));
+    }
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
     const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
-    const bool row_masked = qrow >= tv;
-    const float lse2 = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ls, qrow * 4, 0, 0)) * kLog2e;
 
     RowLane<C> row_lane;
     TrLane<C> tr_lane;
     row_lane.init(0, lane);
     tr_lane.init(0, lane);
-
-    const int row0 = 16 * kStripTiles * strip;
-    stage_direct<C, kStripTiles, kReadShared>(qs, row0, q_lds, kStripTiles, wave, lane_off, a.pitch);
-    stage_direct<C, kStripTiles, kReadShared>(gs, row0, g_lds, kStripTiles, wave, lane_off, a.pitch);
-    stage_direct<C, kStripTiles, kReadShared>(os, row0, o_lds, kStripTiles, wave, lane_off, a.pitch);
-    f32x4 acc[CT];
+    f32x4 acc[QT][CT];
+    float dl[QT], ref[QT];              // ref: minus the row's LSE in the log2 domain, a padded row's -100 taken out of it
+    bool row_masked[QT];
+    uint32_t drop_key[QT];
+    wait_direct();
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) acc[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-    RowOperand<C> qop, gop;
-    float dl = 0.f;
-    // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dP = D * (dO . V^T) and delta = rowsum(dO * O) as before.
-    const uint32_t drop_key = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
-
-    for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
-        if (c0) __syncthreads();
-        stage_direct<C, kStripTiles, kReadShared>(ks, 16 * c0, k_lds, kStripTiles, wave, lane_off, a.pitch);
-        stage_direct<C, kStripTiles, kReadShared>(vs, 16 * c0, v_lds, kStripTiles, wave, lane_off, a.pitch);
-        wait_direct();
-        __syncthreads();
-        if (c0 == 0) {
-            RowOperand<C> oop;
-            read_rows<C>(qop, q_lds + wave * LL::kTileBytes, row_lane);
-            read_rows<C>(gop, g_lds + wave * LL::kTileBytes, row_lane);
-            read_rows<C>(oop, o_lds + wave * LL::kTileBytes, row_lane);
-            dl = xor_sum(dot_lane<DT, C>(gop, oop));        // lane (n, g) holds a quarter of row n's channels
-        }
-        const int nk = min(kStripTiles, tiles - c0);
+    for (int h = 0; h < QT; ++h) {
+        const int qrow = 16 * qt[h] + n;
+        dl[h] = xor_sum(dot_lane<DT, C>(gop[h], oop[h]));   // lane (n, g) holds a quarter of row n's channels
+        row_masked[h] = qrow >= tv;
+        ref[h] = (row_masked[h] ? mask2 : 0.f) - lse_row[h] * kLog2e;
+        // With dropout mask D (0 or 1/(1-p)): O = (D*P) V, so dP = D * (dO . V^T) and delta = rowsum(dO * O) as before.
+        drop_key[h] = DROP ? dropout_row_key((uint64_t)b * T + qrow, a.drop) : 0u;
 #pragma unroll
-        for (int kt = 0; kt < kStripTiles; ++kt) {
+        for (int ct = 0; ct < CT; ++ct) acc[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // one chunk of keys; `whole`: all of its 64 keys exist and count
+    auto chunk = [&](auto whole, int c0, LDS_PTR(char) k_lds, LDS_PTR(char) v_lds) {
+        constexpr bool kWhole = decltype(whole)::value;
+        const int nk = kWhole ? kStripTiles : min(kStripTiles, tiles - c0);
+#pragma unroll
+        for (int kt = 0; kt < kStripTiles; kt += 2) {
             if (kt >= nk) continue;
-            RowOperand<C> kop, vop;
-            read_rows<C>(kop, k_lds + kt * LL::kTileBytes, row_lane);
-            read_rows<C>(vop, v_lds + kt * LL::kTileBytes, row_lane);
-            const f32x4 s = dot_rows_mma<DT, C>(kop, qop);
-            const f32x4 dp = dot_rows_mma<DT, C>(vop, gop);
-            float dsv[4];
+            u32x4 db[QT];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int key = 16 * (c0 + kt) + 4 * g + r;
-                const float z = s[r] * scale2 - lse2 + ((key >= tv || row_masked) ? mask2 : 0.f);
-                const float p = key < T ? __builtin_amdgcn_exp2f(z) : 0.f;
-                float dpr = dp[r];
-                if constexpr (DROP) dpr *= dropout_keeps(drop_key, key, a.drop) ? a.drop.inv_keep : 0.f;
-                dsv[r] = p * (dpr - dl);
+            for (int j = 0; j < 2; ++j) {
+                if (kt + j < nk) {
+                    RowOperand<C> kop, vop;
+                    read_rows<C>(kop, k_lds + (kt + j) * LL::kTileBytes, row_lane);
+                    read_rows<C>(vop, v_lds + (kt + j) * LL::kTileBytes, row_lane);
+#pragma unroll
+                    for (int h = 0; h < QT; ++h) {
+                        const f32x4 s = dot_rows_mma<DT, C>(kop, qop[h]);
+                        const f32x4 dp = dot_rows_mma<DT, C>(vop, gop[h]);
+                        float dsv[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int key = 16 * (c0 + kt + j) + 4 * g + r;
+                            float z = __builtin_fmaf(s[r], scale2, ref[h]);
+                            if constexpr (!kWhole) z += (key >= tv && !row_masked[h]) ? mask2 : 0.f;
+                            const float p = kWhole || key < T ? __builtin_amdgcn_exp2f(z) : 0.f;
+                            float dpr = dp[r];
+                            if constexpr (DROP) dpr *= dropout_keeps(drop_key[h], key, a.drop) ? a.drop.inv_keep : 0.f;
+                            dsv[r] = p * (dpr - dl[h]);
+                        }
+                        db[h][2 * j] = Mma<DT>::pack(dsv[0], dsv[1]);
+                        db[h][2 * j + 1] = Mma<DT>::pack(dsv[2], dsv[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int h = 0; h < QT; ++h) db[h][2 * j] = db[h][2 * j + 1] = 0u;     // against the zeros staged past the sequence
+                }
             }
-            const u32x2 db = {Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
             LDS_PTR(char) blk = k_lds + kt * LL::kTileBytes;
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) acc[ct] = Mma<DT>::k16(read_tr(blk + tr_lane.off[ct]), db, acc[ct]);
-        }
-    }
-    if (qt >= tiles) return;
-    u32x2 qw[CT];
+            for (int ct = 0; ct < CT; ++ct) {
+                const u32x2 k0 = read_tr(blk + tr_lane.off[ct]), k1 = read_tr(blk + LL::kTileBytes + tr_lane.off[ct]);
+                const u32x4 kk = {k0.x, k0.y, k1.x, k1.y};
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[ct], a.scale);
-    store_tile<C>(dqs, qrow * a.pitch, qw, g, stores_whole_lines(a.pitch, C, 0), a.pitch);
-    if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(dl), ds, qrow * 4, 0, 0);
+                for (int h = 0; h < QT; ++h) acc[h][ct] = Mma<DT>::k32(kk, db[h], acc[h][ct]);
+            }
+        }
+    };
+    const int whole_keys = min(T, tv);
+    int at = 0;                                             // byte offset of the chunk's pair of regions: 0 or 2 * kStep
+    auto step = [&](auto whole, int c0) {
+        wait_direct();
+        barrier_lds();      // this chunk has landed, and every wave is done with the one before, whose regions the next takes
+        if (c0 + kStripTiles < tiles) {
+            LDS_PTR(char) next = kv_lds + (at ^ 2 * kStep);
+            stage_direct<C, kStripTiles, kReadShared>(ks, 16 * (c0 + kStripTiles), next, kStripTiles, wave, lane_off, a.pitch);
+            stage_direct<C, kStripTiles, kReadShared>(vs, 16 * (c0 + kStripTiles), next + kStep, kStripTiles, wave, lane_off, a.pitch);
+        }
+        chunk(whole, c0, kv_lds + at, kv_lds + at + kStep);
+        at ^= 2 * kStep;
+    };
+    int c0 = 0;
+    for (; 16 * (c0 + kStripTiles) <= whole_keys; c0 += kStripTiles) step(std::true_type{}, c0);
+    for (; c0 < tiles; c0 += kStripTiles) step(std::false_type{}, c0);
+
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        if (qt[h] >= tiles) break;
+        const int qrow = 16 * qt[h] + n;
+        u32x2 qw[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) qw[ct] = pack_acc<DT>(acc[h][ct], a.scale);
+        store_tile<C>(dqs, qrow * a.pitch, qw, g, stores_whole_lines(a.pitch, C, 0), a.pitch);
+        if (g == 0) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(dl[h]), ds, qrow * 4, 0, 0);
+    }
 }
 
 // =============================================================================
 // Backward, key side: dK and dV
 // =============================================================================
-template <class DT, int C, bool DROP>
+// A workgroup owns 4 * QT key tiles, QT to a wave, whose K and V rows go from memory straight into registers, and
+// walks the queries in chunks of 4 tiles (Q, dO, LSE and delta through LDS, double-buffered).  The score product is
+// taken with Q and K swapped, so that P and dS come out as B operands; dV^T += dO^T P and dK^T += Q^T dS run two
+// query tiles at a time on the 32-deep product.
+template <class DT, int C, bool DROP, int QT>
 __global__ void __launch_bounds__(kThreads)
 global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__restrict__ q, const char *__restrict__ k,
                   const char *__restrict__ v, const char *__restrict__ dout, const float *__restrict__ lse,
@@ -557,15 +606,12 @@ global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__re
     constexpr int CT = C / 16;
     constexpr int kStep = region_bytes<C>(kStripTiles);
     constexpr int kRows = 16 * kStripTiles;                 // rows of a chunk: one lse / delta value each
+    constexpr int kBuf = 2 * kStep + 2 * kRows * 4;         // Q, dO, lse, delta of one chunk
     fetch_args_now(dk, dv, q, k, v, dout, lse, delta, t_valid, items, a.T, a.H, a.strips, a.strips_magic, a.heads_magic,
                    a.pitch, a.scale);
-    extern __shared__ __attribute__((aligned(16))) char smem[];          // 4 * kStep + 2 * kRows * 4 bytes
-    LDS_PTR(char) k_lds = (LDS_PTR(char))smem;
-    LDS_PTR(char) v_lds = k_lds + kStep;
-    LDS_PTR(char) q_lds = v_lds + kStep;
-    LDS_PTR(char) g_lds = q_lds + kStep;                    // dO
-    LDS_PTR(float) lse_lds = (LDS_PTR(float))(g_lds + kStep);
-    LDS_PTR(float) del_lds = lse_lds + kRows;
+    if constexpr (DROP) fetch_args_now(a.drop.threshold, a.drop.seed_lo, a.drop.seed_hi, a.drop.inv_keep);
+    extern __shared__ __attribute__((aligned(16))) char smem[];          // 2 * kBuf bytes
+    LDS_PTR(char) buf_lds = (LDS_PTR(char))smem;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -575,8 +621,6 @@ global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__re
     const int strip = (int)(item - b * a.strips);
     const uint32_t sample = div_by(b, a.H, a.heads_magic);
     const int T = a.T, tiles = (T + 15) >> 4;
-    const int kt_own = kStripTiles * strip + wave;          // this wave's key tile
-    const int key = 16 * kt_own + n;
 
     const int64_t seq_off = (int64_t)b * T * a.pitch;
     const Rsrc qs = make_rsrc(q + seq_off, T * a.pitch), ks = make_rsrc(k + seq_off, T * a.pitch);
@@ -584,78 +628,128 @@ global_dkv_kernel(char *__restrict__ dk, char *__restrict__ dv, const char *__re
     const Rsrc dks = make_rsrc(dk + seq_off, T * a.pitch), dvs = make_rsrc(dv + seq_off, T * a.pitch);
     const Rsrc ls = make_rsrc(lse + (int64_t)b * T, T * 4), ds = make_rsrc(delta + (int64_t)b * T, T * 4);
     const int lane_off = direct_lane_offset<C>(wave, lane, a.pitch, a.pitch);
+    auto stage = [&](int c0, LDS_PTR(char) buf) {           // chunk of queries c0 .. c0 + 3 into one buffer
+        stage_direct<C, kStripTiles, kReadShared>(qs, 16 * c0, buf, kStripTiles, wave, lane_off, a.pitch);
+        stage_direct<C, kStripTiles, kReadShared>(gs, 16 * c0, buf + kStep, kStripTiles, wave, lane_off, a.pitch);
+        if (wave == 0) load_to_lds<4, 0>(ls, buf + 2 * kStep, (16 * c0 + lane) * 4);            // rows past T: zeros
+        if (wave == 1) load_to_lds<4, 0>(ds, buf + 2 * kStep + kRows * 4, (16 * c0 + lane) * 4);
+    };
+    stage(0, buf_lds);
+    int kt_own[QT];                                         // this wave's key tiles
+    RowOperand<C> kop[QT], vop[QT];
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        kt_own[h] = kStripTiles * (QT * strip + h) + wave;
+        load_rows<C, kReadShared>(kop[h], ks, 16 * kt_own[h] * a.pitch, a.pitch, a.pitch, lane);
+        load_rows<C, kReadShared>(vop[h], vs, 16 * kt_own[h] * a.pitch, a.pitch, a.pitch, lane);
+    }
     int tv = T;
     if (t_valid) tv = max(0, min(T, t_valid[sample]));
     const float scale2 = a.scale * kLog2e, mask2 = kMaskValue * kLog2e;
-    const bool col_masked = key >= tv;
 
     RowLane<C> row_lane;
     TrLane<C> tr_lane;
     row_lane.init(0, lane);
     tr_lane.init(0, lane);
-
-    const int row0 = 16 * kStripTiles * strip;
-    stage_direct<C, kStripTiles, kReadShared>(ks, row0, k_lds, kStripTiles, wave, lane_off, a.pitch);
-    stage_direct<C, kStripTiles, kReadShared>(vs, row0, v_lds, kStripTiles, wave, lane_off, a.pitch);
-    f32x4 acck[CT], accv[CT];
+    f32x4 acck[QT][CT], accv[QT][CT];
+    bool keys_count = true;             // all keys of this wave's tiles are valid ones
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) acck[ct] = accv[ct] = f32x4{0.f, 0.f, 0.f, 0.f};
-    RowOperand<C> kop, vop;
-
-    for (int c0 = 0; c0 < tiles; c0 += kStripTiles) {
-        if (c0) __syncthreads();
-        stage_direct<C, kStripTiles, kReadShared>(qs, 16 * c0, q_lds, kStripTiles, wave, lane_off, a.pitch);
-        stage_direct<C, kStripTiles, kReadShared>(gs, 16 * c0, g_lds, kStripTiles, wave, lane_off, a.pitch);
-        if (wave == 0) load_to_lds<4, 0>(ls, (LDS_PTR(char))lse_lds, (16 * c0 + lane) * 4);
-        if (wave == 1) load_to_lds<4, 0>(ds, (LDS_PTR(char))del_lds, (16 * c0 + lane) * 4);
-        wait_direct();
-        __syncthreads();
-        if (c0 == 0) {
-            read_rows<C>(kop, k_lds + wave * LL::kTileBytes, row_lane);
-            read_rows<C>(vop, v_lds + wave * LL::kTileBytes, row_lane);
-        }
-        const int nq = min(kStripTiles, tiles - c0);        // query tiles in this chunk
+    for (int h = 0; h < QT; ++h) {
+        keys_count = keys_count && 16 * kt_own[h] + 16 <= tv;
 #pragma unroll
-        for (int qi = 0; qi < kStripTiles; ++qi) {
+        for (int ct = 0; ct < CT; ++ct) acck[h][ct] = accv[h][ct] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+
+    // one chunk of queries; `whole`: all of its 64 rows exist and count, and so do this wave's keys
+    auto chunk = [&](auto whole, int c0, LDS_PTR(char) buf) {
+        constexpr bool kWhole = decltype(whole)::value;
+        LDS_PTR(char) q_lds = buf;
+        LDS_PTR(char) g_lds = buf + kStep;
+        LDS_PTR(float) lse_lds = (LDS_PTR(float))(buf + 2 * kStep);
+        LDS_PTR(float) del_lds = lse_lds + kRows;
+        const int nq = kWhole ? kStripTiles : min(kStripTiles, tiles - c0);      // query tiles in this chunk
+#pragma unroll
+        for (int qi = 0; qi < kStripTiles; qi += 2) {
             if (qi >= nq) continue;
-            RowOperand<C> qop, gop;
-            read_rows<C>(qop, q_lds + qi * LL::kTileBytes, row_lane);
-            read_rows<C>(gop, g_lds + qi * LL::kTileBytes, row_lane);
-            const f32x4 s = dot_rows_mma<DT, C>(qop, kop);   // [query 4g+r][key n]
-            const f32x4 dp = dot_rows_mma<DT, C>(gop, vop);
-            float p[4], dsv[4];
+            u32x4 pb[QT], db[QT];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int qloc = qi * 16 + 4 * g + r, qrow = 16 * c0 + qloc;
-                const float z = s[r] * scale2 - lse_lds[qloc] * kLog2e + ((col_masked || qrow >= tv) ? mask2 : 0.f);
-                p[r] = qrow < T ? __builtin_amdgcn_exp2f(z) : 0.f;     // rows past the sequence do not exist
-                float f = 1.f;             // dropout: dP is masked, and dV takes the probability as the forward used it
-                if constexpr (DROP)
-                    f = dropout_keeps(dropout_row_key((uint64_t)b * T + qrow, a.drop), key, a.drop) ? a.drop.inv_keep : 0.f;
-                dsv[r] = p[r] * (dp[r] * f - del_lds[qloc]);
-                p[r] *= f;
+            for (int j = 0; j < 2; ++j) {
+                if (qi + j < nq) {
+                    RowOperand<C> qop, gop;
+                    read_rows<C>(qop, q_lds + (qi + j) * LL::kTileBytes, row_lane);
+                    read_rows<C>(gop, g_lds + (qi + j) * LL::kTileBytes, row_lane);
+                    const f32x4 lse4 = *reinterpret_cast<LDS_PTR(f32x4)>(lse_lds + 16 * (qi + j) + 4 * g);
+                    const f32x4 del4 = *reinterpret_cast<LDS_PTR(f32x4)>(del_lds + 16 * (qi + j) + 4 * g);
+#pragma unroll
+                    for (int h = 0; h < QT; ++h) {
+                        const int key = 16 * kt_own[h] + n;
+                        const f32x4 s = dot_rows_mma<DT, C>(qop, kop[h]);        // [query 4g+r][key n]
+                        const f32x4 dp = dot_rows_mma<DT, C>(gop, vop[h]);
+                        float p[4], dsv[4];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int qrow = 16 * (c0 + qi + j) + 4 * g + r;
+                            float z = __builtin_fmaf(s[r], scale2, -kLog2e * lse4[r]);
+                            if constexpr (!kWhole) z += (key >= tv || qrow >= tv) ? mask2 : 0.f;
+                            p[r] = kWhole || qrow < T ? __builtin_amdgcn_exp2f(z) : 0.f;     // rows past the sequence do not exist
+                            float f = 1.f;     // dropout: dP is masked, and dV takes the probability as the forward used it
+                            if constexpr (DROP)
+                                f = dropout_keeps(dropout_row_key((uint64_t)b * T + qrow, a.drop), key, a.drop) ? a.drop.inv_keep : 0.f;
+                            dsv[r] = p[r] * (dp[r] * f - del4[r]);
+                            p[r] *= f;
+                        }
+                        pb[h][2 * j] = Mma<DT>::pack(p[0], p[1]);
+                        pb[h][2 * j + 1] = Mma<DT>::pack(p[2], p[3]);
+                        db[h][2 * j] = Mma<DT>::pack(dsv[0], dsv[1]);
+                        db[h][2 * j + 1] = Mma<DT>::pack(dsv[2], dsv[3]);
+                    }
+                } else {
+#pragma unroll
+                    for (int h = 0; h < QT; ++h) pb[h][2 * j] = pb[h][2 * j + 1] = db[h][2 * j] = db[h][2 * j + 1] = 0u;
+                }
             }
-            const u32x2 pb = {Mma<DT>::pack(p[0], p[1]), Mma<DT>::pack(p[2], p[3])};
-            const u32x2 db = {Mma<DT>::pack(dsv[0], dsv[1]), Mma<DT>::pack(dsv[2], dsv[3])};
             LDS_PTR(char) qtile = q_lds + qi * LL::kTileBytes;
             LDS_PTR(char) gtile = g_lds + qi * LL::kTileBytes;
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
-                accv[ct] = Mma<DT>::k16(read_tr(gtile + tr_lane.off[ct]), pb, accv[ct]);
-                acck[ct] = Mma<DT>::k16(read_tr(qtile + tr_lane.off[ct]), db, acck[ct]);
+                const u32x2 g0 = read_tr(gtile + tr_lane.off[ct]), g1 = read_tr(gtile + LL::kTileBytes + tr_lane.off[ct]);
+                const u32x2 q0 = read_tr(qtile + tr_lane.off[ct]), q1 = read_tr(qtile + LL::kTileBytes + tr_lane.off[ct]);
+                const u32x4 gg = {g0.x, g0.y, g1.x, g1.y}, qq = {q0.x, q0.y, q1.x, q1.y};
+#pragma unroll
+                for (int h = 0; h < QT; ++h) {
+                    accv[h][ct] = Mma<DT>::k32(gg, pb[h], accv[h][ct]);
+                    acck[h][ct] = Mma<DT>::k32(qq, db[h], acck[h][ct]);
+                }
             }
         }
-    }
-    if (kt_own >= tiles) return;
-    u32x2 kw[CT], vw[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        kw[ct] = pack_acc<DT>(acck[ct], a.scale);
-        vw[ct] = pack_acc<DT>(accv[ct], 1.f);
-    }
+    };
+    const int whole_rows = keys_count ? min(T, tv) : 0;
+    int at = 0;
+    auto step = [&](auto whole, int c0) {
+        wait_direct();
+        barrier_lds();      // this chunk has landed, and every wave is done with the one before, whose buffer the next takes
+        if (c0 + kStripTiles < tiles) stage(c0 + kStripTiles, buf_lds + (at ^ kBuf));
+        chunk(whole, c0, buf_lds + at);
+        at ^= kBuf;
+    };
+    int c0 = 0;
+    for (; 16 * (c0 + kStripTiles) <= whole_rows; c0 += kStripTiles) step(std::true_type{}, c0);
+    for (; c0 < tiles; c0 += kStripTiles) step(std::false_type{}, c0);
+
     const bool stream = stores_whole_lines(a.pitch, C, 0);
-    store_tile<C>(dks, key * a.pitch, kw, g, stream, a.pitch);      // rows past T are dropped
-    store_tile<C>(dvs, key * a.pitch, vw, g, stream, a.pitch);
+#pragma unroll
+    for (int h = 0; h < QT; ++h) {
+        if (kt_own[h] >= tiles) break;
+        const int key = 16 * kt_own[h] + n;
+        u32x2 kw[CT], vw[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            kw[ct] = pack_acc<DT>(acck[h][ct], a.scale);
+            vw[ct] = pack_acc<DT>(accv[h][ct], 1.f);
+        }
+        store_tile<C>(dks, key * a.pitch, kw, g, stream, a.pitch);      // rows past T are dropped
+        store_tile<C>(dvs, key * a.pitch, vw, g, stream, a.pitch);
+    }
 }
 
 // =============================================================================
@@ -852,9 +946,6 @@ global_bwd_short_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__re
 }
 
 // ----------------------------------------------------------------------------- launchers
-template <int C> constexpr size_t global_lds(int regions) {
-    return (size_t)regions * region_bytes<C>(kStripTiles) + 2 * 16 * kStripTiles * sizeof(float);
-}
 inline bool global_ok(const Geom &g, GlobalArgs &a, int64_t &items) {
     if (g.C > 128 || g.T > (1 << 28) / g.C) return false;
     const int tiles = (int)((g.T + 15) / 16);
@@ -937,18 +1028,33 @@ int launch_global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q,
             return tiles_max == 4 ? go(global_bwd_short_kernel<DT, C, true, 4, 1>) : go(global_bwd_short_kernel<DT, C, true, 8, 1>);
         return tiles_max == 4 ? go(global_bwd_short_kernel<DT, C, false, 4, 1>) : go(global_bwd_short_kernel<DT, C, false, 8, 1>);
     }
-    auto dq_kern = g.drop.threshold ? global_dq_kernel<DT, C, true> : global_dq_kernel<DT, C, false>;
-    auto dkv_kern = g.drop.threshold ? global_dkv_kernel<DT, C, true> : global_dkv_kernel<DT, C, false>;
-    if (!allow_lds(dq_kern, global_lds<C>(5)) || !allow_lds(dkv_kern, global_lds<C>(4))) return NA1D_ERR_LAUNCH;
-    // the pair of profiling events, if set, spans both kernels
-    note_kernel_as("global_dq_kernel + global_dkv_kernel<%s, %d, %s>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C,
-                   g.drop.threshold ? "true" : "false");
-    launch_kernel_span(1, dq_kern, (unsigned)items, (unsigned)kThreads, global_lds<C>(5), s, (char *)dq, delta, (const char *)q,
-                       (const char *)k, (const char *)v, (const char *)out, (const char *)dout, lse, t_valid, (uint32_t)items, a);
-    launch_kernel_span(2, dkv_kern, (unsigned)items, (unsigned)kThreads, global_lds<C>(4), s, (char *)dk, (char *)dv,
-                       (const char *)q, (const char *)k, (const char *)v, (const char *)dout, lse, delta, t_valid,
-                       (uint32_t)items, a);
-    return launch_status();
+    // two tiles to a wave where that leaves no workgroup half empty and every CU several workgroups
+    const int64_t strips2 = (a.strips + 1) / 2;
+    const bool two = a.strips % 2 == 0 && g.B * strips2 >= 4 * 256 && div_magic_ok(g.B * strips2, strips2);
+    if (two) {
+        a.strips = (int)strips2;
+        a.strips_magic = div_magic(a.strips);
+        items = g.B * strips2;
+    }
+    constexpr size_t dq_lds = 4 * (size_t)region_bytes<C>(kStripTiles);
+    constexpr size_t dkv_lds = 2 * (2 * (size_t)region_bytes<C>(kStripTiles) + 2 * 16 * kStripTiles * sizeof(float));
+    auto go = [&](auto dq_kern, auto dkv_kern) {
+        if (!allow_lds(dq_kern, dq_lds) || !allow_lds(dkv_kern, dkv_lds)) return (int)NA1D_ERR_LAUNCH;
+        // the pair of profiling events, if set, spans both kernels
+        note_kernel_as("global_dq_kernel + global_dkv_kernel<%s, %d, %s, %d>", DT::tag == NA1D_BF16 ? "BF16" : "FP16", C,
+                       g.drop.threshold ? "true" : "false", two ? 2 : 1);
+        launch_kernel_span(1, dq_kern, (unsigned)items, (unsigned)kThreads, dq_lds, s, (char *)dq, delta, (const char *)q,
+                           (const char *)k, (const char *)v, (const char *)out, (const char *)dout, lse, t_valid, (uint32_t)items, a);
+        launch_kernel_span(2, dkv_kern, (unsigned)items, (unsigned)kThreads, dkv_lds, s, (char *)dk, (char *)dv,
+                           (const char *)q, (const char *)k, (const char *)v, (const char *)dout, lse, delta, t_valid,
+                           (uint32_t)items, a);
+        return launch_status();
+    };
+    if (g.drop.threshold)
+        return two ? go(global_dq_kernel<DT, C, true, 2>, global_dkv_kernel<DT, C, true, 2>)
+                   : go(global_dq_kernel<DT, C, true, 1>, global_dkv_kernel<DT, C, true, 1>);
+    return two ? go(global_dq_kernel<DT, C, false, 2>, global_dkv_kernel<DT, C, false, 2>)
+               : go(global_dq_kernel<DT, C, false, 1>, global_dkv_kernel<DT, C, false, 1>);
 }
 
 int global_fwd(void *out, float *lse, const void *q, const void *k, const void *v, const int32_t *t_valid,

@@ -18,6 +18,8 @@ GEOMS = [  # (N, H, T, C): one tile, ragged tiles, several strips and chunks, ev
     # launches of many sequences
     (2, 3, 49, 64), (2, 2, 128, 64), (1, 2, 113, 64), (1, 2, 128, 128), (1, 1, 17, 128), (3, 256, 100, 16),
     (2, 400, 128, 32), (3, 256, 81, 64),
+    # long sequences in a launch large enough for two tiles to a wave (strips in pairs), padded and not
+    (2, 256, 200, 16), (1, 512, 250, 32),
 ]
 
 
@@ -91,7 +93,7 @@ def test_global_attention_rejects_wide_heads():
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
 @pytest.mark.parametrize("geom", [(2, 2, 37, 32), (1, 3, 130, 64), (2, 1, 100, 24), (1, 2, 300, 16), (2, 384, 100, 16),
-                                  (2, 2, 128, 64)],
+                                  (2, 2, 128, 64), (2, 256, 200, 16)],
                          ids=lambda g: "x".join(map(str, g)))
 def test_global_attention_dropout_matches_oracle_with_the_same_mask(geom, dtype):
     N, H, T, C = geom
