@@ -381,8 +381,9 @@ global_fwd_short_kernel(char *__restrict__ out, float *__restrict__ lse, const c
         }
         l[h] = DROP ? xor_sum(part) : 0.f;
     }
-    // O^T = V^T P^T, two key tiles to a 32-deep product (a last single tile: 16-deep).  Without dropout the row sums
-    // come from the same instruction with ones in place of V^T.
+    // O^T = V^T P^T, two key tiles to a 32-deep product.  Without dropout the row sums come from the same instruction
+    // with ones in place of V^T.  An accumulator sees products of one depth only: a 16-deep product that takes the
+    // result of a 32-deep one as its accumulator straight behind it has read stale values here.
     f32x4 o[QT][CT], lsum[QT];
 #pragma unroll
     for (int h = 0; h < QT; ++h) {
@@ -409,16 +410,18 @@ global_fwd_short_kernel(char *__restrict__ out, float *__restrict__ lse, const c
                 for (int h = 0; h < QT; ++h)
                     lsum[h] = Mma<DT>::k32(u32x4{one, one, one, one},
                                            u32x4{pb[h][kt].x, pb[h][kt].y, pb[h][kt + 1].x, pb[h][kt + 1].y}, lsum[h]);
-        } else {
+        } else {                // a last single tile against zeros in the other half: one kind of product per accumulator
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
                 const u32x2 vt = read_tr(blk + tr_lane.off[ct]);
 #pragma unroll
-                for (int h = 0; h < QT; ++h) o[h][ct] = Mma<DT>::k16(vt, pb[h][kt], o[h][ct]);
+                for (int h = 0; h < QT; ++h)
+                    o[h][ct] = Mma<DT>::k32(u32x4{vt.x, vt.y, 0u, 0u}, u32x4{pb[h][kt].x, pb[h][kt].y, 0u, 0u}, o[h][ct]);
             }
             if constexpr (!DROP)
 #pragma unroll
-                for (int h = 0; h < QT; ++h) lsum[h] = Mma<DT>::k16(u32x2{one, one}, pb[h][kt], lsum[h]);
+                for (int h = 0; h < QT; ++h)
+                    lsum[h] = Mma<DT>::k32(u32x4{one, one, 0u, 0u}, u32x4{pb[h][kt].x, pb[h][kt].y, 0u, 0u}, lsum[h]);
         }
         __builtin_amdgcn_sched_barrier(0);
     }
