@@ -96,7 +96,7 @@ wide_fwd_kernel(char *__restrict__ out, float *__restrict__ lse, const char *__r
     v_lane.init(16 * sb - shift, lane);
 
     wait_direct();
-    __syncthreads();
+    barrier_lds();
     float bias[NBV][4];
 #pragma unroll
     for (int vb = 0; vb < NBV; ++vb)
@@ -222,12 +222,14 @@ static_assert(kWideQueryTiles * 16 <= kThreads, "one lane per staged lse row");
 
 struct WideBwdShape {
     int hb, ha, mt;                      // halo query tiles before / after, strip length
+    int kx;                              // key blocks that touch a strip's rows beyond one per tile: 1 unless shift % 16 == 0
 };
 inline WideBwdShape wide_bwd_shape(const WideCover &c) {
     WideBwdShape w;
     w.hb = c.nbv - 1 - (c.shift >> 4);
     w.ha = (c.shift + 15) >> 4;
     w.mt = kWideQueryTiles - w.hb - w.ha;
+    w.kx = w.ha - (c.shift >> 4);
     return w;
 }
 
@@ -250,7 +252,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
     const int qtiles = nt + hb + ha;                        // query-side tiles, <= kWideQueryTiles
     const int ktiles = qtiles + NBV - 1;                    // key-side tiles: whole virtual blocks
     // dynamic LDS (launch_wide_bwd): [K region | V region] starting at the first key of query tile i0 - hb, reused
-    // after pass 1 for the score tiles [(tq * NBV + vb) * 2 + P/dS] and padded to kv_bytes; Q, dO regions of qtiles
+    // after pass 1 for the score tiles of the strip's key blocks [((kp - kp_lo) * NBV + vb) * 2 + P/dS] and padded to kv_bytes; Q, dO regions of qtiles
     // tiles; lse of the query-side rows; bias; d rpb slot sums per wave
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int key_region = region_bytes<C>(ktiles), qry_region = region_bytes<C>(qtiles);
@@ -300,7 +302,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
     tr_lane.init(0, lane);
 
     wait_direct();
-    __syncthreads();
+    barrier_lds();
     float bias[NBV][4];
 #pragma unroll
     for (int vb = 0; vb < NBV; ++vb)
@@ -415,25 +417,31 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
         }
     }
 
-    __syncthreads();                    // every wave is done with K and V: their regions become the score tiles
+    // Pass 2 reads the score tiles of the key blocks that touch the strip's rows, kp_lo .. kp_hi: block vb of query
+    // tile tq is key block q0 + tq + vb, and only those in the range are kept (about half of what pass 1 computed).
+    const int kp_lo = i0 + (shift >> 4), kp_hi = i1 - 1 + ha;
+    barrier_lds();                      // every wave is done with K and V: their regions become the score tiles
 #pragma unroll
     for (int jt = 0; jt < kWideTPW; ++jt) {
         const int tq = wave + jt * kWaves;
         if (tq >= qtiles) continue;
-        LDS_PTR(char) t = sc_lds + tq * NBV * 2 * kScoreTile + n * 32 + g * 8;     // tile[query n][key slots 4g..4g+3]
+        LDS_PTR(char) t = sc_lds + n * 32 + g * 8;          // tile[query n][key slots 4g..4g+3]
 #pragma unroll
-        for (int vb = 0; vb < NBV; ++vb)
+        for (int vb = 0; vb < NBV; ++vb) {
+            const int kp = q0 + tq + vb;
+            if (kp < kp_lo || kp > kp_hi) continue;
 #pragma unroll
-            for (int pd = 0; pd < 2; ++pd) *reinterpret_cast<LDS_PTR(u32x2)>(t + (vb * 2 + pd) * kScoreTile) = sc[jt][vb][pd];
+            for (int pd = 0; pd < 2; ++pd)
+                *reinterpret_cast<LDS_PTR(u32x2)>(t + (((kp - kp_lo) * NBV + vb) * 2 + pd) * kScoreTile) = sc[jt][vb][pd];
+        }
     }
-    __syncthreads();
+    barrier_lds();
 
     // ---------------- pass 2: key blocks of the strip -> dK, dV ----------------
     const int sc_lane = (4 * g + (n >> 2)) * 32 + (n & 3) * 8;       // transposed read of a score tile
     const int row_lo = 16 * i0, row_hi = min(T, 16 * i1);            // rows this strip owns
     const Rsrc dks = make_rsrc(dk + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
     const Rsrc dvs = make_rsrc(dv + in_off + (int64_t)row_lo * in.pitch, (row_hi - row_lo) * in.pitch);
-    const int kp_lo = i0 + (shift >> 4), kp_hi = i1 - 1 + ha;
     const bool whole_lines = stores_whole_lines(in.pitch, C, shift);
     for (int kp = kp_lo + wave; kp <= kp_hi; kp += kWaves) {
         f32x4 acck[CT], accv[CT];
@@ -444,7 +452,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
             const int tq = kp - vb - q0;                    // in [0, qtiles) by the choice of hb and ha
             LDS_PTR(char) qtile = q_lds + tq * LL::kTileBytes;
             LDS_PTR(char) gtile = g_lds + tq * LL::kTileBytes;
-            LDS_PTR(char) stile = sc_lds + (tq * NBV + vb) * 2 * kScoreTile + sc_lane;
+            LDS_PTR(char) stile = sc_lds + ((kp - kp_lo) * NBV + vb) * 2 * kScoreTile + sc_lane;
             const u32x2 pb = read_tr(stile), db = read_tr(stile + kScoreTile);
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) {
@@ -478,7 +486,7 @@ wide_bwd_kernel(char *__restrict__ dq, char *__restrict__ dk, char *__restrict__
 template <int C>
 inline size_t wide_bwd_lds(int nt, int nbv, const WideBwdShape &w, int &kv_bytes) {
     const int qtiles = nt + w.hb + w.ha, ktiles = qtiles + nbv - 1;
-    kv_bytes = std::max(2 * region_bytes<C>(ktiles), qtiles * nbv * 2 * 512);
+    kv_bytes = std::max(2 * region_bytes<C>(ktiles), (nt + w.kx) * nbv * 2 * 512);    // K and V, later the score tiles pass 2 reads
     return (size_t)kv_bytes + (size_t)2 * region_bytes<C>(qtiles) +
            (kThreads + kBiasSlots + kWaves * kWideSlots) * sizeof(float);
 }
