@@ -127,3 +127,50 @@ def test_global_attention_dropout_mask_is_bit_exact():
     out = global_attention(q, q, v.cuda(), 1, scale=1.0, dropout_p=p, seed=seed).cpu()
     keep = O.dropout_keep(B, T, T, p, seed)
     assert torch.equal(out[:, :, :T] != 0, keep) and (out[:, :, T:] == 0).all()
+
+
+FULL_SIZE = [  # (N, H, T, C, dtype, backward): the models' dense layers at their benchmark sizes, and a long backward
+    (256, 4, 100, 64, torch.bfloat16, False), (64, 4, 1000, 64, torch.bfloat16, False),
+    (128, 4, 100, 64, torch.float16, True), (64, 4, 520, 64, torch.bfloat16, True),
+]
+
+
+@pytest.mark.parametrize("case", FULL_SIZE, ids=lambda c: "x".join(map(str, c[:4])) + ("-bwd" if c[5] else ""))
+def test_global_attention_properties_at_full_size(case):
+    """Size-independent properties under a full launch, where every CU holds several workgroups: a slice of the batch
+    run alone gives the same bits as inside the batch (forward and gradients), two runs agree bit for bit, rows of P
+    sum to one (v = 1 gives 1), and the slice agrees with the oracle."""
+    N, H, T, C, dtype, bwd = case
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, 0, 123, dtype, n=4)
+    scale = C ** -0.5
+    t_valid = torch.full((N,), T, dtype=torch.int32)
+    t_valid[N // 2:] = T - T // 3                     # half the samples padded
+    sl = slice(B // 2 - 2 * H, B // 2 + 2 * H)        # two unpadded and two padded samples
+    ns = slice(N // 2 - 2, N // 2 + 2)
+    print("global attention at full size", case, flush=True)
+
+    def run(qq, kk, vv, dd, tv):
+        qd, kd, vd = (t.cuda().requires_grad_(bwd) for t in (qq, kk, vv))
+        out = global_attention(qd, kd, vd, H, t_valid=tv.cuda(), scale=scale)
+        if bwd:
+            out.backward(dd.cuda())
+            return out.detach(), qd.grad, kd.grad, vd.grad
+        return (out.detach(),)
+
+    full = run(q, k, v, do, t_valid)
+    again = run(q, k, v, do, t_valid)
+    alone = run(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), do[sl].contiguous(), t_valid[ns])
+    for name, a, b, c in zip(("O", "dQ", "dK", "dV"), full, again, alone):
+        assert torch.equal(a, b), name + ": two runs differ"
+        assert torch.equal(a[sl], c), name + ": a slice alone differs from the slice inside the batch"
+    pad = T - t_valid[ns]
+    qf, kf, vf = q[sl].float(), k[sl].float(), v[sl].float()
+    want_o, _, _ = O.global_forward(qf, kf, vf, scale, pad, H)
+    assert O.rel_l2(alone[0].float().cpu(), want_o) < TOL[dtype], "O"
+    if bwd:
+        wq, wk, wv = O.global_backward(qf, kf, vf, do[sl].float(), scale, pad, H)
+        for name, got, ref in (("dQ", alone[1], wq), ("dK", alone[2], wk), ("dV", alone[3], wv)):
+            assert O.rel_l2(got.float().cpu(), ref) < TOL[dtype], name
+    ones = run(q, k, torch.ones_like(v), do, t_valid)[0]
+    assert (ones.float() - 1).abs().max() < 2e-2

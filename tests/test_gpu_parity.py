@@ -417,6 +417,45 @@ def test_config2_forward_backward_fp16():
         assert O.rel_l2(got.float(), ref) < 2e-3, name
 
 
+FULL_LAUNCHES = [  # (N, H, T, C, W, L, dtype): the configurations' shapes and a wide window, forward and backward
+    (128, 16, 100, 16, 27, 13, torch.float16), (128, 8, 300, 32, 15, 7, torch.float16),
+    (64, 16, 1000, 16, 27, 13, torch.bfloat16), (128, 8, 300, 32, 65, 32, torch.float16),
+]
+
+
+@pytest.mark.parametrize("case", FULL_LAUNCHES, ids=lambda c: "x".join(map(str, c[:6])))
+def test_full_launches_are_deterministic_and_batch_invariant(case):
+    """Under a launch that fills the card (every CU holds several workgroups, copies and matrix instructions of
+    different workgroups interleave) the kernels give the same bits twice, and a slice of the batch run alone gives
+    the bits it has inside the batch: outputs and the gradients of q, k, v (d rpb, summed with float atomics by
+    default, is left out).  The slice is checked against the oracle."""
+    N, H, T, C, W, L, dtype = case
+    B = N * H
+    q, k, v, do = make_inputs(B, T, C, W, 7, dtype, n=4, scale=C ** -0.5)
+    rpb = torch.randn(H, W, generator=torch.Generator().manual_seed(3)) * 0.5
+    t_valid = torch.full((N,), T, dtype=torch.int32)
+    t_valid[N // 2:] = T - T // 4
+    sl, ns = slice(B // 2 - 2 * H, B // 2 + 2 * H), slice(N // 2 - 2, N // 2 + 2)
+    print("full launch", case, flush=True)
+
+    def run(qq, kk, vv, dd, tv):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (qq, kk, vv))
+        out = na1d_fused(qd, kd, vd, W, L, rpb=rpb.cuda(), t_valid=tv.cuda(), num_heads=H)
+        out.backward(dd.cuda())
+        return out.detach(), qd.grad, kd.grad, vd.grad
+
+    full = run(q, k, v, do, t_valid)
+    again = run(q, k, v, do, t_valid)
+    alone = run(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous(), do[sl].contiguous(), t_valid[ns])
+    for name, a, b, c in zip(("O", "dQ", "dK", "dV"), full, again, alone):
+        assert torch.equal(a, b), name + ": two runs differ"
+        assert torch.equal(a[sl], c), name + ": a slice alone differs from the slice inside the batch"
+    pad = T - t_valid[ns]
+    qf, kf, vf = q[sl].float(), k[sl].float(), v[sl].float()
+    want, _, _ = O.na1d_forward(qf, kf, vf, W, L, rpb=rpb, padding=pad, num_heads=H)
+    assert O.rel_l2(alone[0].float().cpu(), want) < TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
 def test_model_shape_properties_at_full_size(dtype):
     """cfg3's NA shape (B 4096, T 100, C 16, W 27): size-independent properties
