@@ -456,6 +456,47 @@ def test_full_launches_are_deterministic_and_batch_invariant(case):
     assert O.rel_l2(alone[0].float().cpu(), want) < TOL[dtype]
 
 
+@pytest.mark.parametrize("case", [(256, 16, 100, 16, 27, 13, torch.bfloat16), (128, 8, 300, 32, 15, 7, torch.float16)],
+                         ids=lambda c: "x".join(map(str, c[:6])))
+def test_full_launches_in_the_projection_layout_and_through_the_two_call_api(case):
+    """The same two properties for the operator on the qkv projection's output (head-group forward, strided backward)
+    and for the un-fused functions of the reference's API, at full size."""
+    N, H, T, C, W, L, dtype = case
+    g = torch.Generator().manual_seed(11)
+    qkv = (torch.randn(N, T, 3, H, C, generator=g) * 0.5).to(dtype)
+    do = torch.randn(N, T, H * C, generator=g).to(dtype)
+    rpb = torch.randn(H, W, generator=g) * 0.5
+    ns = slice(N // 2 - 2, N // 2 + 2)
+    print("full launch, projection layout", case, flush=True)
+
+    def run(x, dd):
+        xd = x.cuda().requires_grad_(True)
+        out = na1d_fused_qkv(xd, W, L, rpb=rpb.cuda(), scale=C ** -0.5)
+        out.backward(dd.cuda())
+        return out.detach(), xd.grad
+
+    full, again, alone = run(qkv, do), run(qkv, do), run(qkv[ns].contiguous(), do[ns].contiguous())
+    for name, a, b, c in zip(("O", "dqkv"), full, again, alone):
+        assert torch.equal(a, b), name + ": two runs differ"
+        assert torch.equal(a[ns], c), name + ": a slice alone differs from the slice inside the batch"
+
+    QK, AV = nattn.getNA1dFunction(C, 1, dtype)
+    q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3).reshape(N * H, T, C).contiguous() for i in range(3))
+    sl = slice(ns.start * H, ns.stop * H)
+
+    def chain(qq, kk, vv):
+        qd, kd, vd = (t.cuda().requires_grad_(True) for t in (qq, kk, vv))
+        attn = QK.apply(qd, kd, W, L, 1)
+        out = AV.apply(torch.softmax(attn, -1), vd, W, L, 1)
+        out.float().square().sum().backward()
+        return attn.detach(), out.detach(), qd.grad, kd.grad, vd.grad
+
+    full, again, alone = chain(q, k, v), chain(q, k, v), chain(q[sl].contiguous(), k[sl].contiguous(), v[sl].contiguous())
+    for name, a, b, c in zip(("S", "O", "dQ", "dK", "dV"), full, again, alone):
+        assert torch.equal(a, b), name + ": two runs differ"
+        assert torch.equal(a[sl], c), name + ": a slice alone differs from the slice inside the batch"
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=["bf16", "fp16"])
 def test_model_shape_properties_at_full_size(dtype):
     """cfg3's NA shape (B 4096, T 100, C 16, W 27): size-independent properties
