@@ -8,7 +8,6 @@
 namespace na1d {
 namespace mfma {
 
-constexpr int kMaxWideBlocks = 6;
 constexpr int kBiasSlots = 96;   // W <= 80, padded
 
 // Blocks and shift of a wide window; 0 blocks if the shape is not covered.
