@@ -20,6 +20,8 @@ GEOMS = [  # (N, H, T, C): one tile, ragged tiles, several strips and chunks, ev
     (2, 400, 128, 32), (3, 256, 81, 64),
     # long sequences in a launch large enough for two tiles to a wave (strips in pairs), padded and not
     (2, 256, 200, 16), (1, 512, 250, 32),
+    # long sequences with a sample that is padding from its first row on
+    (3, 2, 150, 32), (3, 1, 200, 64),
 ]
 
 
