@@ -372,9 +372,10 @@ def wide_record(lib, clock, name, steps, warmup, device):
 
 
 def global_record(lib, clock, name, steps, warmup, device):
-    """Dense attention at one of the models' shapes.  These kernels are bound by the matrix cores and LDS, not by HBM:
-    the record gives TFLOP/s against the dense 16-bit matrix-core peak, counting 4*T*T*C flop per sequence forward
-    (Q.K^T and P.V) and 10*T*T*C backward (five products of that size), next to the bytes moved."""
+    """Dense attention at one of the models' shapes.  At a thousand rows a sequence the kernels are bound by the matrix
+    and vector instructions, at a hundred they are short memory-bound launches: the record gives TFLOP/s against the
+    dense 16-bit matrix-core peak, counting 4*T*T*C flop per sequence forward (Q.K^T and P.V) and 10*T*T*C backward
+    (five products of that size), next to the bytes moved and their rate."""
     import torch
     from na1d_amd import _lib
     w = GLOBAL_WORKLOADS[name]
