@@ -22,6 +22,8 @@ GEOMS = [  # (N, H, T, C): one tile, ragged tiles, several strips and chunks, ev
     (2, 256, 200, 16), (1, 512, 250, 32),
     # long sequences with a sample that is padding from its first row on
     (3, 2, 150, 32), (3, 1, 200, 64),
+    # long sequences of heads narrower than the kernel's width
+    (2, 2, 140, 24), (1, 2, 260, 104),
 ]
 
 
