@@ -988,9 +988,10 @@ int launch_global_fwd(void *out, float *lse, const void *q, const void *k, const
             return small ? go(global_fwd_short_kernel<DT, C, true, 4, 1>) : go(global_fwd_short_kernel<DT, C, true, 8, 2>);
         return small ? go(global_fwd_short_kernel<DT, C, false, 4, 1>) : go(global_fwd_short_kernel<DT, C, false, 8, 2>);
     }
-    // two query tiles to a wave where that still leaves every CU several workgroups and no workgroup half empty
+    // two query tiles to a wave where that still leaves every CU several workgroups and at most one workgroup in seven
+    // or more half empty
     const int64_t strips2 = (a.strips + 1) / 2;
-    const bool two = a.strips % 2 == 0 && g.B * strips2 >= 4 * 256 && div_magic_ok(g.B * strips2, strips2);
+    const bool two = (a.strips % 2 == 0 || a.strips >= 7) && g.B * strips2 >= 4 * 256 && div_magic_ok(g.B * strips2, strips2);
     if (two) {
         a.strips = (int)strips2;
         a.strips_magic = div_magic(a.strips);
@@ -1031,9 +1032,9 @@ int launch_global_bwd(void *dq, void *dk, void *dv, float *delta, const void *q,
             return tiles_max == 4 ? go(global_bwd_short_kernel<DT, C, true, 4, 1>) : go(global_bwd_short_kernel<DT, C, true, 8, 1>);
         return tiles_max == 4 ? go(global_bwd_short_kernel<DT, C, false, 4, 1>) : go(global_bwd_short_kernel<DT, C, false, 8, 1>);
     }
-    // two tiles to a wave where that leaves no workgroup half empty and every CU several workgroups
+    // two tiles to a wave where that leaves every CU several workgroups and at most one workgroup in seven or more half empty
     const int64_t strips2 = (a.strips + 1) / 2;
-    const bool two = a.strips % 2 == 0 && g.B * strips2 >= 4 * 256 && div_magic_ok(g.B * strips2, strips2);
+    const bool two = (a.strips % 2 == 0 || a.strips >= 7) && g.B * strips2 >= 4 * 256 && div_magic_ok(g.B * strips2, strips2);
     if (two) {
         a.strips = (int)strips2;
         a.strips_magic = div_magic(a.strips);
